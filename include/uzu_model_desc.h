@@ -110,7 +110,16 @@ typedef enum {
      * (head_norm_epsilon, no weights), the heads are concatenated, multiplied by silu(gate h) and projected.  q and k are rotated (use_rope) and k is multiplied
      * by key_scale behind its rotation.  Fields: num_heads, head_dim, value_head_dim, retention_decay, qkv_projection (rows: queries | keys | values | gate,
      * n = 2 heads head_dim + 2 heads value_head_dim), out_projection (k = heads * value_head_dim). */
-    UZU_MIXER_RETENTION = 3
+    UZU_MIXER_RETENTION = 3,
+    /* Gated linear recurrent unit behind a short causal convolution (f32-stream designs): two branches of lru_width channels from ONE packed projection
+     * (qkv_projection rows: gate branch | recurrent branch, n = 2 lru_width, with out_biases).  The recurrent branch runs through a per-channel causal convolution
+     * (dn_kernel_size taps, dn_conv_weights f32 [lru_width, taps], the last tap weighs the current position, dn_conv_biases f32 [lru_width]) giving u; the channels
+     * are split into lru_blocks equal blocks with two square gate matrices each (lru_gate_weights bf16 [blocks][2 bw][bw], bw = lru_width / lru_blocks: the
+     * recurrence gate's rows, then the input gate's; lru_gate_biases f32 [blocks][2 bw]): r = sigmoid(A_b u_b + a_b), i = sigmoid(B_b u_b + b_b).  With
+     * a = exp(-lru_decay_rate r softplus(lru_lambda)) the state is S_t = a S_(t-1) + sqrt(1 - a^2) i u (f32 [lru_width], zero in front of position 0) and the
+     * mixer's result out_projection(S_t * gelu_tanh(gate branch)) (k = lru_width).  Gates, decays and the state are f32 in both precisions; the sequence state
+     * is S and the convolution's last taps - 1 inputs. */
+    UZU_MIXER_GATED_LRU = 4
 } uzu_mixer_kind;
 
 /* config/rope/*.rs -- every AnyRoPEConfig variant (encodable_block/mixer/attention/rope.rs:13-114) */
@@ -271,8 +280,36 @@ typedef struct {
     float key_scale;             /* keys are multiplied by it behind their rotation; 0 = 1 */
     float head_norm_epsilon;     /* UZU_MIXER_RETENTION: epsilon of the per-head RMS division */
     const float* retention_decay; /* UZU_MIXER_RETENTION: f32 [num_heads] */
-    uint32_t reserved4;
-    uint32_t reserved6;
+    /* UZU_MIXER_LATENT_ATTENTION with a rotated key part: the down projection yields latent_rank + latent_rope_dim numbers per token -- the latent (normed) and ONE
+     * rotated key part shared by all heads (not normed); a query head is [head_dim | latent_rope_dim] wide and its last latent_rope_dim coordinates turn with the
+     * same rotation (use_rope + rope_index, rope_interleaved); score = attention_scale (<q_plain, W_up_k c> + <q_rot, k_rot>).  The cache row is [latent | rotated part].
+     * latent_packed: the down projection's rows stand behind the queries in qkv_projection (latent_down absent); has_gate then adds num_heads rows behind them:
+     * head a's result is multiplied by sigmoid(gate row a . h). */
+    uint32_t latent_rope_dim;
+    uint32_t latent_packed;
+    uint32_t rope_interleaved;   /* the rotation pairs coordinates (2i, 2i + 1) instead of (i, i + dims / 2) */
+    /* UZU_MIXER_GATED_LRU (see uzu_mixer_kind) */
+    uint32_t lru_width;
+    uint32_t lru_blocks;
+    float lru_decay_rate;
+    const uint16_t* lru_gate_weights; /* bf16 [blocks][2 bw][bw] */
+    const float* lru_gate_biases;     /* f32 [blocks][2 bw] */
+    const float* lru_lambda;          /* f32 [lru_width] */
+    /* Layer scale (f32-stream designs): the mixer's result (behind post_mixer_norm) is multiplied element by element by layer_scale_mixer before it joins the
+     * stream, the MLP's (behind post_mlp_norm) by layer_scale_mlp; f32 [model_dim] or NULL.  In an f32-stream design post_mixer_norm / post_mlp_norm, query_norm /
+     * key_norm (scales [head_dim], before the rotation) and UZU_NORM_STATISTICS norms (RMS, scales + scale_offset) are honoured as well. */
+    const float* layer_scale_mixer;
+    const float* layer_scale_mlp;
+    /* A gated dense MLP in an f32-stream design (mlp_plain == 0): up_projection rows [up ; gate], hidden = clamp-gated product with the constants of
+     * moe.{silu_alpha, gate_clip_*, up_clip_*, up_offset} (mlp_kind stays UZU_MLP_DENSE, no other field of `moe` is read). */
+    /* Per-layer token input in an f32-stream design (has_ple, ple_dim, ple_gate, ple_projection, ple_norm with the model's ple_token_embedding): behind the MLP
+     * x <- x + norm(projection(gelu_tanh(gate x) * e)), e = columns [ple_slice ple_dim, (ple_slice + 1) ple_dim) of the token's row of the side table. */
+    uint32_t ple_slice;
+    /* Weight sharing between layer runs (a looped stack): weights_of_layer = j + 1 makes this run use run j's tensors (its own pointers are ignored; scalars must
+     * agree); every run keeps its own sequence state.  0 = its own. */
+    uint32_t weights_of_layer;
+    /* Re-entry of the stream: before this run x <- W [x ; x0] with x0 the embedding rows (n = model_dim, k = 2 model_dim); absent = none */
+    uzu_linear_desc stream_reentry;
 } uzu_layer_desc;
 
 typedef struct {

@@ -5,4 +5,4 @@ host-side mirror of the reference's backend trait surface, ``engine.py`` the mod
 ``desc.py`` / ``synthetic.py`` model description and synthetic format-exact weights.
 Compute only ever runs through ``lib/libuzu_hip.so`` on an AMD GPU; there is no CPU fallback.
 """
-__all__ = ["backend", "desc", "engine", "synthetic", "lazolix", "relulix", "serving"]
+__all__ = ["backend", "desc", "engine", "synthetic", "lazolix", "relulix", "begasun", "serving"]

@@ -333,7 +333,10 @@ uzu_status uzu_hip_model_create_tp(uzu_hip_context* ctx, const uzu_model_desc* d
         UZU_UNSUPPORTED(desc->layers[l].mixer_kind == UZU_MIXER_LATENT_ATTENTION || desc->layers[l].mixer_kind == UZU_MIXER_RETENTION || desc->layers[l].parallel_block ||
                         desc->layers[l].score_soft_cap != 0.0f || desc->layers[l].unit_sink || desc->layers[l].key_scale != 0.0f || desc->layers[l].token_shift || desc->layers[l].depth_weights || desc->layers[l].mlp_plain ||
                         desc->layers[l].no_mlp || desc->layers[l].pre_mixer_norm.kind != UZU_NORM_STATISTICS || desc->layers[l].pre_mlp_norm.kind != UZU_NORM_STATISTICS ||
-                        (desc->layers[l].mlp_kind == UZU_MLP_MOE && desc->layers[l].moe.routing != UZU_MOE_ROUTE_TOPK_LOGITS),
+                        (desc->layers[l].mlp_kind == UZU_MLP_MOE && desc->layers[l].moe.routing != UZU_MOE_ROUTE_TOPK_LOGITS) ||
+                        desc->layers[l].mixer_kind == UZU_MIXER_GATED_LRU || desc->layers[l].latent_rope_dim || desc->layers[l].latent_packed || desc->layers[l].rope_interleaved ||
+                        desc->layers[l].layer_scale_mixer || desc->layers[l].layer_scale_mlp || desc->layers[l].weights_of_layer || desc->layers[l].stream_reentry.weights ||
+                        desc->layers[l].ple_slice,
                         "model_create: layer %u uses a mechanism of the f32-stream designs (set uzu_model_desc::f32_stream)", l);
     (void)hipSetDevice(ctx->device);
     auto* m = new uzu_hip_model();

@@ -16,6 +16,12 @@
 // f32 state per sequence (k_retention.hip), top-k routed experts with clamped gates, a scaled embedding and an untied read-out.  Each is chosen per layer by the
 // description's fields, so a model may mix them.
 //
+// A third family (Begasun) adds: RMS norms with a weight vector stored around zero in front of AND behind every sublayer, a layer scale on each sublayer's result, a
+// per-layer token input (a slice of a second token table, gated by the stream), a gated dense block with clamps, layer runs that share an earlier run's tensors with
+// a re-entry projection of [stream ; embedding rows] (a looped stack; every run keeps its own sequence state), latent attention whose cache row carries one rotated
+// key part for all heads (interleaved pairs, scaled frequencies) with a sigmoid gate per head, per-head query / key norms on the cached-key attention, and a
+// gated linear recurrent unit behind a short convolution (k_gated_lru.hip).
+//
 // Precisions: `bf16_products` (default) rounds the activation operand of every matrix product to bf16 and keeps the latent cache in bf16; UZU_MODEL_FULL_F32
 // makes every product a true f32 product and the cache f32.  Everything else is f32 either way.
 #include <algorithm>
@@ -36,6 +42,7 @@ struct Stream32 {
     float *slots = nullptr, *xin = nullptr, *normed = nullptr, *q = nullptr, *ckv = nullptr, *qlat = nullptr, *ctx = nullptr, *attn = nullptr, *hid = nullptr;
     int32_t* moe_ids = nullptr;
     float* moe_w = nullptr;
+    float *tmp = nullptr, *y1 = nullptr, *lru_u = nullptr, *lru_g = nullptr, *side_g = nullptr; // a sublayer's result in front of its post norm; [up | gate] of a gated dense block; LRU input / gates; token-input gate
     float *moe_y1 = nullptr, *moe_y2 = nullptr; // grouped expert form: [max_rows * top][2 ff] and [max_rows * top][d]
     uint32_t *moe_perm = nullptr, *moe_slot_pos = nullptr, *moe_offsets = nullptr, *moe_cursor = nullptr;
     float *out_normed = nullptr, *logits = nullptr;
@@ -51,6 +58,10 @@ struct Stream32 {
         float *token_shift = nullptr, *depth_weights = nullptr, *selection_bias = nullptr;
         float alpha1 = 0.f, alpha2 = 0.f;
         float* decay = nullptr; // retention: f32 [heads]
+        float *ls1 = nullptr, *ls2 = nullptr; // layer scales f32 [d]
+        uint16_t* lru_gate_w = nullptr;       // gated LRU: bf16 [blocks][2 bw][bw]
+        float *lru_gate_b = nullptr, *lru_lambda = nullptr;
+        DLinear reentry_a, reentry_b; // the re-entry projection's halves: on the stream, on the embedding rows
     };
     std::vector<Layer> layers;
     float alpha_out = 0.f;
@@ -117,6 +128,10 @@ void run_norm(Enc& e, const DNorm& N, uint32_t kind, float alpha, const float* x
         RUN("rms_norm_rows", (size_t)rows * d * 8, k::rms_norm_rows(s, x, out, nullptr, alpha, N.eps, row_index, rows, d));
         return;
     }
+    if (kind == UZU_NORM_STATISTICS) { // RMS with a weight vector (+ offset)
+        RUN("rms_norm_rows", (size_t)rows * d * 8, k::rms_norm_rows(s, x, out, N.scales, 1.0f, N.eps, row_index, rows, d, N.offset));
+        return;
+    }
     k::DynTanhParams np{};
     np.x = x, np.out = out, np.scales = N.scales, np.biases = N.biases, np.alpha = alpha, np.row_index = row_index, np.rows = rows, np.d = d;
     RUN("dyn_tanh_norm", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
@@ -156,6 +171,7 @@ uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs,
             const uzu_hip_state::Layer& own = seqs[i].st->layers[src];
             const size_t at = (size_t)l * S.max_seqs + i;
             if (h.mixer_kind == UZU_MIXER_ATTENTION) cache_ptrs[at] = own.cache_k, cache2_ptrs[at] = own.cache_v;
+            else if (h.mixer_kind == UZU_MIXER_GATED_LRU) cache_ptrs[at] = own.ssm_state, cache2_ptrs[at] = own.conv_state;
             else if (h.mixer_kind == UZU_MIXER_RETENTION) cache_ptrs[at] = own.ret_state;
             else cache_ptrs[at] = own.latent;
             shift_ptrs[at] = seqs[i].st->layers[l].shift_prev;
@@ -187,13 +203,22 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     const uint32_t bf = S.full_f32 ? 0u : 1u;
     RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d, m->d.input_scale));
     const float* cur = S.slots; // what the layer about to run reads: X_0, then the depth mix of the layer before
+    uint32_t max_count = 0;
+    for (uint32_t c : counts) max_count = std::max(max_count, c);
     for (uint32_t l = 0; l < nl; ++l) {
         DLayer& L = m->layers[l];
         const Stream32::Layer& X = S.layers[l];
         const uzu_layer_desc& h = L.d;
         float* slot = S.slots + (size_t)(l + 1) * slot_stride; // X_(l+1): the layer's own result
         void* const* caches = S.d_cache_ptrs + (size_t)l * S.max_seqs;
-        if (h.pre_mixer_norm.kind == UZU_NORM_RMS_SCALAR) {
+        if (X.reentry_a.w) { // x <- W [x ; x0]: the two halves of W on the stream and on the embedding rows, summed
+            run_linear(e, lin(S, X.reentry_a, cur, S.xin, rows));
+            k::LinearF32Params b = lin(S, X.reentry_b, S.slots, S.xin, rows);
+            b.residual = S.xin, b.ldr = d;
+            run_linear(e, b);
+            cur = S.xin;
+        }
+        if (h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH) {
             run_norm(e, L.pre_mixer, h.pre_mixer_norm.kind, X.alpha1, cur, S.normed, rows, d, nullptr);
         } else { // dynamic-tanh norm + token shift
             k::DynTanhParams np{};
@@ -203,13 +228,28 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         }
         const uint32_t H = h.num_heads, hd = h.head_dim, vd = h.value_head_dim, rank = h.latent_rank;
         run_linear(e, lin(S, L.qkv, S.normed, S.q, rows)); // the packed projection of the mixer (queries first)
-        if (h.mixer_kind == UZU_MIXER_ATTENTION) {
+        if (h.mixer_kind == UZU_MIXER_GATED_LRU) {
+            const uint32_t w = h.lru_width, bw = w / h.lru_blocks;
+            k::GatedLruParams gp{};
+            gp.branches = S.q, gp.ld = L.qkv.n, gp.x_col = w, gp.u = S.lru_u, gp.gates = S.lru_g, gp.out = S.attn, gp.conv_w = L.conv_w, gp.conv_b = L.conv_b, gp.gate_b = X.lru_gate_b;
+            gp.lambda = X.lru_lambda, gp.rate = h.lru_decay_rate, gp.states = (float* const*)caches, gp.conv_states = (float* const*)(S.d_cache2_ptrs + (size_t)l * S.max_seqs);
+            gp.spans = S.d_spans, gp.row_seq = S.d_row_seq, gp.nseq = nseq, gp.rows = rows, gp.width = w, gp.blocks = h.lru_blocks, gp.taps = h.dn_kernel_size, gp.max_count = max_count;
+            RUN("lru_conv", (size_t)rows * w * 4 * (gp.taps + 1), k::lru_conv(s, gp));
+            {   // both gates of every block in one batched product; what enters the recurrence is never rounded: true f32 products in both precisions
+                k::LinearF32Params p{};
+                p.x = S.lru_u, p.w = X.lru_gate_w, p.y = S.lru_g, p.rows = rows, p.n = 2 * bw, p.k = bw, p.ldx = w, p.ldy = 2 * w, p.batch = h.lru_blocks;
+                p.x_batch = bw, p.w_batch = (size_t)2 * bw * bw, p.y_batch = 2 * bw, p.bf16_products = 0;
+                run_linear(e, p);
+            }
+            RUN("lru_scan", (size_t)rows * w * 20, k::lru_scan(s, gp));
+        } else if (h.mixer_kind == UZU_MIXER_ATTENTION) {
             const uint32_t G = h.num_groups, ldq = L.qkv.n;
             void* const* vcaches = S.d_cache2_ptrs + (size_t)l * S.max_seqs;
             k::RopeAppendParams rp{};
             rp.qkv = S.q, rp.ld = ldq, rp.k_col = H * hd, rp.v_col = H * hd + G * hd, rp.heads = H, rp.kv_heads = h.is_kv_sharing ? 0u : G, rp.dim = hd, rp.vdim = vd;
             rp.rope_dim = h.use_rope ? L.rope_dim : 0u, rp.cosines = L.rope_cos, rp.sines = L.rope_sin, rp.key_scale = h.key_scale != 0.0f ? h.key_scale : 1.0f;
             rp.key_caches = caches, rp.value_caches = vcaches, rp.cache_bf16 = bf, rp.spans = S.d_spans, rp.row_seq = S.d_row_seq, rp.rows = rows;
+            rp.q_norm = L.qn.present ? L.qn.scales : nullptr, rp.k_norm = L.kn.present && !h.is_kv_sharing ? L.kn.scales : nullptr, rp.norm_eps = L.qn.present ? L.qn.eps : L.kn.eps;
             RUN("rope_append", (size_t)rows * ldq * 8, k::rope_append(s, rp));
             k::WindowAttentionParams ap{};
             ap.q = S.q, ap.ldq = ldq, ap.out = S.attn, ap.key_caches = caches, ap.value_caches = vcaches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans;
@@ -235,37 +275,62 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             RUN("retention", (size_t)rows * ldq * 4 + (size_t)nseq * H * hd * vd * 8, k::retention(s, tp));
             RUN("head_rms_gate", (size_t)rows * H * vd * 12, k::head_rms_gate(s, S.attn, S.q + 2 * H * hd + H * vd, ldq, h.head_norm_epsilon, rows, H, vd));
         } else {
-        if (!h.is_kv_sharing) {
-            run_linear(e, lin(S, L.lat_down, S.normed, S.ckv, rows));
-            RUN("latent_norm_append", (size_t)rows * rank * 6,
-                k::latent_norm_append(s, S.ckv, L.lat_norm.scales, L.lat_norm.eps, caches, bf, S.d_spans, S.d_row_seq, rows, rank));
+        // rd: the rotated key part every head shares; the cache row is [latent | rotated part] (kw wide), a query head [plain | rotated] (qw wide)
+        const uint32_t rd = h.latent_rope_dim, kw = rank + rd, qw = hd + rd, ldq = L.qkv.n;
+        if (!h.is_kv_sharing && !h.latent_packed) run_linear(e, lin(S, L.lat_down, S.normed, S.ckv, rows));
+        if (!rd && !h.latent_packed) {
+            if (!h.is_kv_sharing)
+                RUN("latent_norm_append", (size_t)rows * rank * 6,
+                    k::latent_norm_append(s, S.ckv, L.lat_norm.scales, L.lat_norm.eps, caches, bf, S.d_spans, S.d_row_seq, rows, rank));
+        } else {
+            k::LatentRopeAppendParams lp{};
+            lp.x = h.latent_packed ? S.q : S.ckv, lp.ldx = h.latent_packed ? ldq : L.lat_down.n, lp.c_col = h.latent_packed ? H * qw : 0, lp.rank = rank, lp.rope_dim = rd;
+            lp.scales = L.lat_norm.scales, lp.eps = L.lat_norm.eps, lp.caches = h.is_kv_sharing ? nullptr : caches, lp.cache_bf16 = bf, lp.heads = H, lp.q_width = qw;
+            lp.qlat = rd ? S.qlat : nullptr, lp.cosines = L.rope_cos, lp.sines = L.rope_sin, lp.interleaved = h.rope_interleaved, lp.spans = S.d_spans, lp.row_seq = S.d_row_seq, lp.rows = rows;
+            if (h.latent_packed) { // the rotated query parts are read from the packed rows; a separate down projection leaves them in S.q as well
+                RUN("latent_rope_append", (size_t)rows * (kw * 6 + H * rd * 8), k::latent_rope_append(s, lp));
+            } else {
+                k::LatentRopeAppendParams cp = lp; // cache rows from the down projection's rows, query parts from the query rows
+                cp.qlat = nullptr;
+                if (!h.is_kv_sharing) RUN("latent_rope_append", (size_t)rows * kw * 6, k::latent_rope_append(s, cp));
+                if (rd) {
+                    k::LatentRopeAppendParams qp = lp;
+                    qp.x = S.q, qp.ldx = ldq, qp.c_col = 0, qp.caches = nullptr;
+                    RUN("latent_rope_append", (size_t)rows * H * rd * 8, k::latent_rope_append(s, qp));
+                }
+            }
         }
-        {   // the head's key projection folded into the query: qlat[r, h, :] = W_up_k[h]^T q[r, h, :]
+        {   // the head's key projection folded into the query: qlat[r, h, :rank] = W_up_k[h]^T q[r, h, :hd]
             k::LinearF32Params p{};
-            p.x = S.q, p.w = X.up_keys_t, p.y = S.qlat, p.rows = rows, p.n = rank, p.k = hd, p.ldx = H * hd, p.ldy = H * rank, p.batch = H;
-            p.x_batch = hd, p.w_batch = (size_t)rank * hd, p.y_batch = rank, p.bf16_products = bf;
+            p.x = S.q, p.w = X.up_keys_t, p.y = S.qlat, p.rows = rows, p.n = rank, p.k = hd, p.ldx = ldq, p.ldy = H * kw, p.batch = H;
+            p.x_batch = qw, p.w_batch = (size_t)rank * hd, p.y_batch = kw, p.bf16_products = bf;
             run_linear(e, p);
         }
         {
             k::LatentAttentionParams ap{};
             ap.qlat = S.qlat, ap.out = S.ctx, ap.caches = caches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans, ap.row_seq = S.d_row_seq;
-            ap.rows = rows, ap.heads = H, ap.rank = rank, ap.window = h.sliding_window_size;
+            ap.rows = rows, ap.heads = H, ap.rank = kw, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd);
             ap.nseq = nseq;
             // decode-sized passes: spread a tile's key blocks over workgroups (a constant of the layer, so that a captured step stays valid as the context grows)
             const uint32_t keys = h.sliding_window_size ? h.sliding_window_size : m->d.max_context_length;
             if (rows <= 4 * S.max_seqs && rows * H <= 4096) ap.splits = std::min<uint32_t>(32, (keys + 31) / 32), ap.split_ws = S.att_ws, ap.split_ws_bytes = S.att_ws_bytes;
             for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] * H + 127) / 128;
-            RUN("latent_attention", (size_t)rows * H * rank * 8, k::latent_attention(s, ap));
+            RUN("latent_attention", (size_t)rows * H * kw * 8, k::latent_attention(s, ap));
         }
-        {   // the head's value projection on the weighted latent sum: attn[r, h, :] = W_up_v[h] ctx[r, h, :]
+        {   // the head's value projection on the weighted latent sum (the rotated columns of the sum are not read): attn[r, h, :] = W_up_v[h] ctx[r, h, :rank],
+            // times the head's sigmoid gate where the layer has one
             k::LinearF32Params p{};
-            p.x = S.ctx, p.w = (const uint16_t*)L.lat_up_v.w, p.y = S.attn, p.rows = rows, p.n = vd, p.k = rank, p.ldx = H * rank, p.ldy = H * vd, p.batch = H;
-            p.x_batch = rank, p.w_batch = (size_t)vd * rank, p.y_batch = vd, p.bf16_products = bf;
+            p.x = S.ctx, p.w = (const uint16_t*)L.lat_up_v.w, p.y = S.attn, p.rows = rows, p.n = vd, p.k = rank, p.ldx = H * kw, p.ldy = H * vd, p.batch = H;
+            p.x_batch = kw, p.w_batch = (size_t)vd * rank, p.y_batch = vd, p.bf16_products = bf;
+            if (h.has_gate) p.gate = S.q + H * qw + (h.latent_packed ? kw : 0), p.ldgate = ldq;
             run_linear(e, p);
         }
         } // latent attention
-        {   // X_(l+1) = input + out projection
+        if (L.post_mixer.present) { // the mixer's result joins the stream behind its own norm (and the layer scale)
+            run_linear(e, lin(S, L.out, S.attn, S.tmp, rows));
+            RUN("rms_norm_add_rows", (size_t)rows * d * 12, k::rms_norm_add_rows(s, S.tmp, cur, slot, L.post_mixer.scales, L.post_mixer.offset, X.ls1, L.post_mixer.eps, rows, d));
+        } else { // X_(l+1) = input + out projection
             k::LinearF32Params p = lin(S, L.out, S.attn, slot, rows);
             p.residual = cur, p.ldr = d;
             run_linear(e, p);
@@ -295,13 +360,30 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
                         k::moe_experts_down_combine(s, S.hid, S.normed, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
                 }
             } else {
-                k::LinearF32Params up = lin(S, L.up, S.normed, S.hid, rows);
-                up.act = 1;
-                run_linear(e, up);
-                k::LinearF32Params down = lin(S, L.down, S.hid, slot, rows);
-                down.residual = slot, down.ldr = d;
-                run_linear(e, down);
+                if (h.mlp_plain) {
+                    k::LinearF32Params up = lin(S, L.up, S.normed, S.hid, rows);
+                    up.act = 1;
+                    run_linear(e, up);
+                } else { // gated: [up ; gate] rows of one projection, then the clamped gate product
+                    run_linear(e, lin(S, L.up, S.normed, S.y1, rows));
+                    RUN("gated_act_rows", (size_t)rows * h.hidden_dim * 12, k::gated_act_rows(s, S.y1, S.hid, rows, h.hidden_dim, expert_act(h.moe)));
+                }
+                if (L.post_mlp.present) {
+                    run_linear(e, lin(S, L.down, S.hid, S.tmp, rows));
+                    RUN("rms_norm_add_rows", (size_t)rows * d * 12, k::rms_norm_add_rows(s, S.tmp, slot, slot, L.post_mlp.scales, L.post_mlp.offset, X.ls2, L.post_mlp.eps, rows, d));
+                } else {
+                    k::LinearF32Params down = lin(S, L.down, S.hid, slot, rows);
+                    down.residual = slot, down.ldr = d;
+                    run_linear(e, down);
+                }
             }
+        }
+        if (h.has_ple) { // the per-layer token input: x <- x + norm(projection(gelu(gate x) * the token's slice of the side table))
+            run_linear(e, lin(S, L.ple_gate, slot, S.side_g, rows));
+            RUN("side_gate_mul", (size_t)rows * h.ple_dim * 10, k::side_gate_mul(s, S.side_g, d_tokens, (const uint16_t*)m->ple_token_embedding.w, m->ple_token_embedding.k,
+                                                                              h.ple_slice * h.ple_dim, m->ple_token_embedding.n, rows, h.ple_dim));
+            run_linear(e, lin(S, L.ple_projection, S.side_g, S.tmp, rows));
+            RUN("rms_norm_add_rows", (size_t)rows * d * 12, k::rms_norm_add_rows(s, S.tmp, slot, slot, L.ple_norm.scales, L.ple_norm.offset, nullptr, L.ple_norm.eps, rows, d));
         }
         if (X.depth_weights) {
             RUN("depth_mix", (size_t)rows * d * 4 * (l + 3), k::depth_mix(s, S.slots, slot_stride, X.depth_weights, h.num_depth_weights, S.xin, rows, d));
@@ -315,7 +397,9 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     S.last_logit_rows = 0;
     if (n_out) {
         run_norm(e, m->output_norm, m->d.output_norm.kind, S.alpha_out, cur, S.out_normed, n_out, d, S.d_out_rows);
-        run_linear(e, lin(S, m->d.tied_embeddings ? m->embedding : m->output_embedding, S.out_normed, S.logits, n_out));
+        k::LinearF32Params head = lin(S, m->d.tied_embeddings ? m->embedding : m->output_embedding, S.out_normed, S.logits, n_out);
+        if (m->d.logit_scale != 1.0f) head.y_scale = m->d.logit_scale; // (0 = a description that never set it)
+        run_linear(e, head);
         S.last_logit_rows = n_out;
     }
     if (e.st != UZU_OK) return e.st;
@@ -390,41 +474,90 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     UZU_REQUIRE(desc->tied_embeddings || (desc->output_embedding.method == UZU_QUANT_NONE && desc->output_embedding.weights && desc->output_embedding.n == desc->vocab_size &&
                                           desc->output_embedding.k == d && !desc->output_embedding.out_biases),
                 "model_create: an untied read-out of an f32-stream design is a full-precision matrix [vocab, model_dim]");
-    auto norm_ok = [](const uzu_norm_desc& n) { return n.present && ((n.kind == UZU_NORM_DYNAMIC_TANH && n.scales) || n.kind == UZU_NORM_RMS_SCALAR); };
-    UZU_REQUIRE(norm_ok(desc->output_norm), "model_create: an f32-stream design ends in a dynamic-tanh norm or an RMS norm with one gain");
-    UZU_UNSUPPORTED(desc->has_ple || desc->embedding_norm.present || desc->logit_soft_cap != 0.0f || desc->logit_scale != 1.0f,
-                    "model_create: decoder options of the bf16-stream families on an f32-stream design");
+    auto rms_vec = [](const uzu_norm_desc& n) { return n.present && n.kind == UZU_NORM_STATISTICS && n.scales && !n.subtract_mean && !n.biases; };
+    auto norm_ok = [&](const uzu_norm_desc& n) { return n.present && ((n.kind == UZU_NORM_DYNAMIC_TANH && n.scales) || n.kind == UZU_NORM_RMS_SCALAR || rms_vec(n)); };
+    UZU_REQUIRE(norm_ok(desc->output_norm), "model_create: an f32-stream design ends in a dynamic-tanh norm or an RMS norm (one gain, or a weight vector)");
+    UZU_UNSUPPORTED(desc->embedding_norm.present || desc->logit_soft_cap != 0.0f, "model_create: decoder options of the bf16-stream families on an f32-stream design");
+    if (desc->has_ple) { // the side table alone: a layer's token input is its slice of the token's row
+        UZU_UNSUPPORTED(desc->ple_model_projection.weights || desc->ple_projection_norm.present, "model_create: an f32-stream design's per-layer token input has no model projection");
+        UZU_REQUIRE(desc->ple_dim && desc->ple_token_embedding.weights && desc->ple_token_embedding.method == UZU_QUANT_NONE && desc->ple_token_embedding.n == desc->ple_vocab_size &&
+                    desc->ple_vocab_size >= desc->vocab_size && desc->ple_token_embedding.k % desc->ple_dim == 0,
+                    "model_create: the side table is a full-precision matrix [>= vocab, slices * ple_dim]");
+    }
     auto full = [](const uzu_linear_desc& L, uint32_t n, uint32_t kk) { return L.weights && L.method == UZU_QUANT_NONE && L.n == n && L.k == kk && !L.input_signs && !L.output_signs && !L.lora_rank; };
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = desc->layers[l];
-        UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION && h.mixer_kind != UZU_MIXER_ATTENTION && h.mixer_kind != UZU_MIXER_RETENTION,
-                        "model_create: layer %u: an f32-stream design's mixer is latent attention, attention over cached keys and values, or retention", l);
-        UZU_REQUIRE(norm_ok(h.pre_mixer_norm), "model_create: layer %u needs a dynamic-tanh or one-gain RMS pre-mixer norm", l);
+        UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION && h.mixer_kind != UZU_MIXER_ATTENTION && h.mixer_kind != UZU_MIXER_RETENTION && h.mixer_kind != UZU_MIXER_GATED_LRU,
+                        "model_create: layer %u: an f32-stream design's mixer is latent attention, attention over cached keys and values, retention, or a gated linear recurrent unit", l);
+        UZU_REQUIRE(norm_ok(h.pre_mixer_norm), "model_create: layer %u needs a dynamic-tanh or RMS pre-mixer norm", l);
         UZU_UNSUPPORTED(h.token_shift && h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH, "model_create: layer %u: the token shift follows a dynamic-tanh norm", l);
+        UZU_REQUIRE(!h.post_mixer_norm.present || rms_vec(h.post_mixer_norm), "model_create: layer %u: a post-mixer norm is an RMS norm with a weight vector", l);
+        UZU_REQUIRE(!h.post_mlp_norm.present || (rms_vec(h.post_mlp_norm) && !h.no_mlp && h.mlp_kind != UZU_MLP_MOE && !h.parallel_block),
+                    "model_create: layer %u: a post-MLP norm is an RMS norm with a weight vector behind a dense block", l);
+        UZU_REQUIRE((!h.layer_scale_mixer || h.post_mixer_norm.present) && (!h.layer_scale_mlp || h.post_mlp_norm.present), "model_create: layer %u: a layer scale follows a post norm", l);
+        UZU_UNSUPPORTED(h.has_post_layer_scalar || h.normalize_values || h.is_non_causal, "model_create: layer %u: layer options of the bf16-stream families", l);
+        if (h.weights_of_layer) {
+            UZU_REQUIRE(h.weights_of_layer - 1 < l, "model_create: layer %u uses the tensors of run %u, which does not precede it", l, h.weights_of_layer - 1);
+            const uzu_layer_desc& src = desc->layers[h.weights_of_layer - 1];
+            UZU_REQUIRE(!src.weights_of_layer && src.mixer_kind == h.mixer_kind && src.qkv_projection.n == h.qkv_projection.n && src.out_projection.k == h.out_projection.k &&
+                        src.hidden_dim == h.hidden_dim && src.no_mlp == h.no_mlp && src.mlp_kind == h.mlp_kind && src.has_ple == h.has_ple && !h.is_kv_sharing && !src.is_kv_sharing &&
+                        (src.stream_reentry.weights != nullptr) == (h.stream_reentry.weights != nullptr),
+                        "model_create: layer %u: a run that shares tensors has the shapes and options of the run that owns them", l);
+        }
+        if (h.stream_reentry.weights) {
+            UZU_REQUIRE(full(h.stream_reentry, d, 2 * d), "model_create: layer %u: the re-entry projection is a full-precision matrix [model_dim, 2 model_dim]", l);
+            UZU_UNSUPPORTED(l > 0 && desc->layers[l - 1].depth_weights, "model_create: layer %u: a re-entry projection behind a depth mix", l);
+        }
+        if (h.has_ple) {
+            UZU_REQUIRE(desc->has_ple && h.ple_dim == desc->ple_dim && (h.ple_slice + 1) * h.ple_dim <= desc->ple_token_embedding.k && full(h.ple_gate, h.ple_dim, d) &&
+                        full(h.ple_projection, d, h.ple_dim) && rms_vec(h.ple_norm) && h.ple_activation == UZU_ACT_GELU_APPROX,
+                        "model_create: layer %u: the token input needs the model's side table, its slice, gate [ple_dim, model_dim], projection [model_dim, ple_dim], a weight-vector RMS norm and the tanh gelu", l);
+        }
+        if (h.mixer_kind == UZU_MIXER_GATED_LRU) {
+            const uint32_t w = h.lru_width;
+            UZU_REQUIRE(w && h.lru_blocks && w % h.lru_blocks == 0 && h.dn_kernel_size >= 1 && h.dn_kernel_size <= 64, "model_create: layer %u: lru_width in lru_blocks equal blocks, 1 .. 64 taps", l);
+            UZU_REQUIRE(full(h.qkv_projection, 2 * w, d) && full(h.out_projection, d, w) && h.dn_conv_weights && h.lru_gate_weights && h.lru_lambda,
+                        "model_create: layer %u: the recurrent unit's packed projection [2 lru_width, model_dim], out projection [model_dim, lru_width], convolution, gates and lambda", l);
+            UZU_UNSUPPORTED(h.is_kv_sharing || h.sliding_window_size || h.has_sinks || h.unit_sink || h.score_soft_cap != 0.0f || h.use_rope || h.has_gate,
+                            "model_create: layer %u: attention options on a recurrent layer", l);
+        } else {
         UZU_REQUIRE(h.num_heads && h.head_dim && h.value_head_dim, "model_create: layer %u: heads / head_dim / value_head_dim", l);
         UZU_REQUIRE(full(h.out_projection, d, h.num_heads * h.value_head_dim), "model_create: layer %u: the out projection must be a full-precision matrix [model_dim, heads * value_head_dim]", l);
+        }
         if (h.use_rope) {
             const uzu_rope_desc& R = desc->num_ropes ? desc->ropes[h.rope_index < desc->num_ropes ? h.rope_index : 0] : desc->rope;
-            UZU_REQUIRE(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION && (!desc->num_ropes || h.rope_index < desc->num_ropes) && R.kind != UZU_ROPE_NONE && R.head_dim && R.head_dim % 2 == 0 &&
-                        R.head_dim <= h.head_dim, "model_create: layer %u: its rotation must turn an even number of at most head_dim coordinates", l);
+            const bool latent = h.mixer_kind == UZU_MIXER_LATENT_ATTENTION;
+            UZU_REQUIRE((!desc->num_ropes || h.rope_index < desc->num_ropes) && R.kind != UZU_ROPE_NONE && R.head_dim && R.head_dim % 2 == 0 &&
+                        (latent ? R.head_dim == h.latent_rope_dim : R.head_dim <= h.head_dim),
+                        "model_create: layer %u: its rotation must turn an even number of at most head_dim coordinates (latent attention: exactly the rotated key part)", l);
+            UZU_UNSUPPORTED(h.rope_interleaved && !latent, "model_create: layer %u: interleaved pairs are the latent attention's rotation", l);
         }
+        UZU_REQUIRE(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION || (h.latent_rope_dim != 0) == (h.use_rope != 0), "model_create: layer %u: a rotated key part and its rotation come together", l);
         if (h.mixer_kind == UZU_MIXER_LATENT_ATTENTION) {
-            UZU_REQUIRE(h.latent_rank && h.latent_rank <= k::kLatentMaxRank, "model_create: layer %u: latent_rank (<= %u)", l, k::kLatentMaxRank);
-            UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim, d) && full(h.latent_up_keys, h.num_heads * h.head_dim, h.latent_rank) &&
-                        full(h.latent_up_values, h.num_heads * h.value_head_dim, h.latent_rank),
-                        "model_create: layer %u: query / latent up projections must be full-precision matrices of the configured shapes", l);
+            const uint32_t rd = h.latent_rope_dim, kw = h.latent_rank + rd, qn = h.num_heads * (h.head_dim + rd);
+            UZU_REQUIRE(h.latent_rank && kw <= k::kLatentMaxRank, "model_create: layer %u: latent_rank (+ the rotated part <= %u)", l, k::kLatentMaxRank);
+            UZU_REQUIRE(full(h.latent_up_keys, h.num_heads * h.head_dim, h.latent_rank) && full(h.latent_up_values, h.num_heads * h.value_head_dim, h.latent_rank),
+                        "model_create: layer %u: latent up projections must be full-precision matrices of the configured shapes", l);
+            if (h.latent_packed) {
+                UZU_REQUIRE(!h.is_kv_sharing && !h.latent_down.weights && full(h.qkv_projection, qn + kw + (h.has_gate ? h.num_heads : 0), d) && h.latent_norm.present && h.latent_norm.scales,
+                            "model_create: layer %u: the packed projection is queries | down projection | gates [heads (head_dim + rope) + rank + rope (+ heads), model_dim], with the latent norm", l);
+            } else {
+                UZU_REQUIRE(full(h.qkv_projection, qn + (h.has_gate ? h.num_heads : 0), d), "model_create: layer %u: the query projection must be a full-precision matrix of the configured shape", l);
+            }
             if (h.is_kv_sharing) {
                 UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the latents of layer %u, which does not precede it", l, h.kv_source_layer_index);
                 const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
-                UZU_REQUIRE(src.mixer_kind == UZU_MIXER_LATENT_ATTENTION && !src.is_kv_sharing && src.latent_rank == h.latent_rank,
+                UZU_REQUIRE(src.mixer_kind == UZU_MIXER_LATENT_ATTENTION && !src.is_kv_sharing && src.latent_rank == h.latent_rank && src.latent_rope_dim == rd,
                             "model_create: layer %u: the source layer %u must own latents of the same rank", l, h.kv_source_layer_index);
-            } else {
-                UZU_REQUIRE(full(h.latent_down, h.latent_rank, d) && h.latent_norm.present && h.latent_norm.scales, "model_create: layer %u owns its latents: down projection + latent norm required", l);
+            } else if (!h.latent_packed) {
+                UZU_REQUIRE(full(h.latent_down, kw, d) && h.latent_norm.present && h.latent_norm.scales, "model_create: layer %u owns its latents: down projection + latent norm required", l);
             }
         } else if (h.mixer_kind == UZU_MIXER_ATTENTION) {
             UZU_REQUIRE(h.num_groups && h.num_heads % h.num_groups == 0, "model_create: layer %u: %u query heads on %u key / value heads", l, h.num_heads, h.num_groups);
-            UZU_UNSUPPORTED(h.has_gate || h.query_norm.present || h.key_norm.present || h.normalize_values || h.is_non_causal,
-                            "model_create: layer %u: gate / head norms / non-causal masks are options of the bf16-stream attention", l);
+            UZU_UNSUPPORTED(h.has_gate, "model_create: layer %u: an output gate is an option of the bf16-stream attention and of latent attention", l);
+            UZU_REQUIRE((!h.query_norm.present || h.query_norm.scales) && (!h.key_norm.present || h.key_norm.scales) &&
+                        (!h.query_norm.present || !h.key_norm.present || h.query_norm.epsilon == h.key_norm.epsilon),
+                        "model_create: layer %u: query / key norms carry weights [head_dim] and one epsilon", l);
             if (h.is_kv_sharing) {
                 UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the cache of layer %u, which does not precede it", l, h.kv_source_layer_index);
                 const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
@@ -435,7 +568,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
                 UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim + h.num_groups * (h.head_dim + h.value_head_dim), d),
                             "model_create: layer %u: the packed projection must be a full-precision matrix [heads head_dim + groups (head_dim + value_head_dim), model_dim]", l);
             }
-        } else {
+        } else if (h.mixer_kind == UZU_MIXER_RETENTION) {
             UZU_REQUIRE(full(h.qkv_projection, 2 * h.num_heads * h.head_dim + 2 * h.num_heads * h.value_head_dim, d) && !h.qkv_projection.out_biases,
                         "model_create: layer %u: a retention layer's packed projection is queries | keys | values | gate without biases", l);
             UZU_REQUIRE(h.retention_decay, "model_create: layer %u: retention without its decays", l);
@@ -455,9 +588,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
                             (M.num_routed_experts == 0 || (M.expert_hidden_dim && M.w13 && M.w2)) && M.gating_sel == 2 && !M.up_biases && !M.down_biases,
                             "model_create: layer %u: routed SiLU-gated experts without biases, with their router and expert tensors", l);
                 UZU_REQUIRE(M.routing == UZU_MOE_ROUTE_SCORES || (!M.num_identity_experts && !M.selection_bias), "model_create: layer %u: identity experts and selection biases belong to score routing", l);
+            } else if (h.mlp_plain) {
+                UZU_REQUIRE(h.activation == UZU_ACT_RELU_SQUARED && full(h.up_projection, h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim),
+                            "model_create: layer %u: the plain dense block is down(relu(up x + b)^2) + b with full-precision matrices", l);
             } else {
-                UZU_REQUIRE(h.mlp_plain && h.activation == UZU_ACT_RELU_SQUARED && full(h.up_projection, h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim),
-                            "model_create: layer %u: the dense block is down(relu(up x + b)^2) + b with full-precision matrices", l);
+                UZU_REQUIRE(h.activation == UZU_ACT_SILU && h.hidden_dim && full(h.up_projection, 2 * h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim) && !h.parallel_block,
+                            "model_create: layer %u: the gated dense block is down(act(gate) * (up + offset)) with full-precision matrices [up ; gate] and [model_dim, hidden]", l);
             }
         }
     }
@@ -484,14 +620,61 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     S.max_rows = m->chunk, S.max_seqs = m->max_seqs;
     m->layers.resize(nl);
     S.layers.resize(nl);
-    uint32_t w_q = 0, w_rank = 0, w_lat = 0, w_attn = 0, w_hid = 0, w_top = 1, w_moe = 0, w_routed = 0;
+    uint32_t w_q = 0, w_rank = 0, w_lat = 0, w_attn = 0, w_hid = 0, w_top = 1, w_moe = 0, w_routed = 0, w_lru = 0, w_side = 0, w_y1 = 0;
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = desc->layers[l];
         DLayer& L = m->layers[l];
         Stream32::Layer& X = S.layers[l];
+        uint32_t kw_l = h.latent_rank + h.latent_rope_dim;
+        w_q = std::max(w_q, h.qkv_projection.n), w_rank = std::max(w_rank, h.latent_down.n ? h.latent_down.n : kw_l), w_lat = std::max(w_lat, h.num_heads * kw_l);
+        w_attn = std::max(w_attn, std::max(h.num_heads * h.value_head_dim, h.lru_width)), w_lru = std::max(w_lru, h.lru_width), w_side = std::max(w_side, h.has_ple ? h.ple_dim : 0u);
+        if (!h.no_mlp && h.mlp_kind != UZU_MLP_MOE) w_hid = std::max(w_hid, h.hidden_dim), w_y1 = std::max(w_y1, h.mlp_plain ? 0u : 2 * h.hidden_dim);
+        if (h.weights_of_layer) { // the tensors of an earlier run: its device pointers, this run's own scalars; nothing is uploaded twice
+            L = m->layers[h.weights_of_layer - 1];
+            X = S.layers[h.weights_of_layer - 1];
+            L.d = h;
+            L.last_reader = l;
+            if (!h.no_mlp && h.mlp_kind == UZU_MLP_MOE) {
+                const uzu_moe_desc& M = h.moe;
+                w_hid = std::max<uint32_t>(w_hid, M.num_active_experts * M.expert_hidden_dim), w_top = std::max(w_top, M.num_active_experts);
+                w_moe = std::max(w_moe, M.num_active_experts * 2 * M.expert_hidden_dim), w_routed = std::max(w_routed, M.num_routed_experts);
+            }
+            continue;
+        }
         L.d = h;
         L.last_reader = l;
         TRY(upload_norm(m, h.pre_mixer_norm, d, &L.pre_mixer));
+        TRY(upload_norm(m, h.post_mixer_norm, d, &L.post_mixer));
+        if (h.layer_scale_mixer) TRY(upload(m, h.layer_scale_mixer, (size_t)d * 4, &X.ls1));
+        if (h.layer_scale_mlp) TRY(upload(m, h.layer_scale_mlp, (size_t)d * 4, &X.ls2));
+        if (h.stream_reentry.weights) { // [d, 2 d] -> the half on the stream and the half on the embedding rows (bf16 bits move)
+            const uint16_t* src = (const uint16_t*)h.stream_reentry.weights;
+            std::vector<uint16_t> a((size_t)d * d), b((size_t)d * d);
+            for (uint32_t n = 0; n < d; ++n) {
+                memcpy(&a[(size_t)n * d], src + (size_t)n * 2 * d, (size_t)d * 2);
+                memcpy(&b[(size_t)n * d], src + (size_t)n * 2 * d + d, (size_t)d * 2);
+            }
+            X.reentry_a.n = X.reentry_b.n = d, X.reentry_a.k = X.reentry_b.k = d;
+            TRY(upload(m, a.data(), a.size() * 2, &X.reentry_a.w));
+            TRY(upload(m, b.data(), b.size() * 2, &X.reentry_b.w));
+        }
+        if (h.has_ple) {
+            TRY(upload_linear(m, h.ple_gate, &L.ple_gate));
+            TRY(upload_linear(m, h.ple_projection, &L.ple_projection));
+            TRY(upload_norm(m, h.ple_norm, d, &L.ple_norm));
+        }
+        if (h.mixer_kind == UZU_MIXER_ATTENTION) {
+            TRY(upload_norm(m, h.query_norm, h.head_dim, &L.qn));
+            TRY(upload_norm(m, h.key_norm, h.head_dim, &L.kn));
+        }
+        if (h.mixer_kind == UZU_MIXER_GATED_LRU) {
+            const size_t w = h.lru_width, bw = w / h.lru_blocks;
+            TRY(upload(m, h.dn_conv_weights, w * h.dn_kernel_size * 4, &L.conv_w));
+            if (h.dn_conv_biases) TRY(upload(m, h.dn_conv_biases, w * 4, &L.conv_b));
+            TRY(upload(m, h.lru_gate_weights, 2 * w * bw * 2, &X.lru_gate_w));
+            if (h.lru_gate_biases) TRY(upload(m, h.lru_gate_biases, 2 * w * 4, &X.lru_gate_b));
+            TRY(upload(m, h.lru_lambda, w * 4, &X.lru_lambda));
+        }
         X.alpha1 = h.pre_mixer_norm.alpha;
         TRY(upload_linear(m, h.qkv_projection, &L.qkv));
         TRY(upload_linear(m, h.out_projection, &L.out));
@@ -512,7 +695,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             TRY(upload(m, t.data(), t.size() * 2, &X.up_keys_t));
         }
         if (!h.is_kv_sharing) {
-            TRY(upload_linear(m, h.latent_down, &L.lat_down));
+            if (!h.latent_packed) TRY(upload_linear(m, h.latent_down, &L.lat_down));
             TRY(upload_norm(m, h.latent_norm, h.latent_rank, &L.lat_norm));
         }
         } // latent attention
@@ -525,6 +708,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         if (h.depth_weights) TRY(upload(m, h.depth_weights, (size_t)h.num_depth_weights * 4, &X.depth_weights));
         if (!h.no_mlp) {
             if (!h.parallel_block) TRY(upload_norm(m, h.pre_mlp_norm, d, &L.pre_mlp));
+            TRY(upload_norm(m, h.post_mlp_norm, d, &L.post_mlp));
             X.alpha2 = h.pre_mlp_norm.alpha;
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
@@ -542,12 +726,10 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             } else {
                 TRY(upload_linear(m, h.up_projection, &L.up));
                 TRY(upload_linear(m, h.down_projection, &L.down));
-                w_hid = std::max(w_hid, h.hidden_dim);
             }
         }
-        w_q = std::max(w_q, h.qkv_projection.n), w_rank = std::max(w_rank, h.latent_rank), w_lat = std::max(w_lat, h.num_heads * h.latent_rank);
-        w_attn = std::max(w_attn, h.num_heads * h.value_head_dim);
     }
+    if (desc->has_ple) TRY(upload_linear(m, desc->ple_token_embedding, &m->ple_token_embedding, true));
     if (!desc->tied_embeddings) TRY(upload_linear(m, desc->output_embedding, &m->output_embedding));
     {   // one table pair per distinct rotation; a layer points at its own
         const uint32_t n_ropes = desc->num_ropes ? desc->num_ropes : (desc->rope.kind != UZU_ROPE_NONE ? 1u : 0u);
@@ -585,6 +767,13 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     TRY(need_f32(m, R * w_lat, &S.ctx));
     TRY(need_f32(m, R * w_attn, &S.attn));
     TRY(need_f32(m, R * (w_hid ? w_hid : 1), &S.hid));
+    TRY(need_f32(m, R * d, &S.tmp));
+    if (w_y1) TRY(need_f32(m, R * w_y1, &S.y1));
+    if (w_lru) {
+        TRY(need_f32(m, R * w_lru, &S.lru_u));
+        TRY(need_f32(m, R * 2 * w_lru, &S.lru_g));
+    }
+    if (w_side) TRY(need_f32(m, R * w_side, &S.side_g));
     TRY(need_f32(m, R * w_top, &S.moe_w));
     if (w_moe && !S.full_f32) { // workspaces of the grouped expert form (bf16 products only)
         void* q = nullptr;
@@ -608,6 +797,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     {
         uint32_t hmax = 0;
         for (uint32_t l = 0; l < nl; ++l) hmax = std::max(hmax, desc->layers[l].num_heads);
+        if (!hmax) hmax = 1;
         const uint32_t few = std::min<uint32_t>(4 * S.max_seqs, 4096 / hmax ? 4096 / hmax : 1);
         S.att_ws_bytes = std::max(k::latent_attention_split_ws_bytes(few, hmax, 256, 32), k::window_attention_split_ws_bytes(few, hmax, 16));
         TRY(need_f32(m, S.att_ws_bytes / 4, &S.att_ws));
@@ -650,6 +840,11 @@ uzu_status s32_state_layer(uzu_hip_model* m, uzu_hip_state* st, uint32_t l) {
     if (h.mixer_kind == UZU_MIXER_RETENTION) { // read only behind position 0, where the kernel starts from zeros: no fill needed
         UZU_PROPAGATE(state_alloc(st, (size_t)h.num_heads * h.head_dim * h.value_head_dim * 4, &p, false));
         st->layers[l].ret_state = (float*)p;
+    } else if (h.mixer_kind == UZU_MIXER_GATED_LRU) { // the state and the convolution's last taps - 1 inputs; both read only behind position 0
+        UZU_PROPAGATE(state_alloc(st, (size_t)h.lru_width * 4, &p, false));
+        st->layers[l].ssm_state = (float*)p;
+        UZU_PROPAGATE(state_alloc(st, (size_t)h.lru_width * (h.dn_kernel_size > 1 ? h.dn_kernel_size - 1 : 1) * 4, &p, false));
+        st->layers[l].conv_state = (float*)p;
     } else if (!h.is_kv_sharing) { // rows are written before they are read (the append precedes the core in every pass)
         if (h.mixer_kind == UZU_MIXER_ATTENTION) {
             UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.num_groups * h.head_dim * elem, &p, false));
@@ -657,7 +852,7 @@ uzu_status s32_state_layer(uzu_hip_model* m, uzu_hip_state* st, uint32_t l) {
             UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.num_groups * h.value_head_dim * elem, &p, false));
             st->layers[l].cache_v = p;
         } else {
-            UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * h.latent_rank * elem, &p, false));
+            UZU_PROPAGATE(state_alloc(st, (size_t)m->max_positions * (h.latent_rank + h.latent_rope_dim) * elem, &p, false));
             st->layers[l].latent = p;
         }
     }

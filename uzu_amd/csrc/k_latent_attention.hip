@@ -39,6 +39,51 @@ __global__ void __launch_bounds__(256) latent_norm_append_kernel(const float* x,
     }
 }
 
+// a workgroup per row: wave 0 norms the latent and writes [latent | rotated key part] to the cache, all waves turn the query heads' rotated parts into qlat
+__global__ void __launch_bounds__(256) latent_rope_append_kernel(LatentRopeAppendParams p) {
+    const uint32_t r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t q = p.row_seq[r];
+    const SeqSpan sp = p.spans[q];
+    const uint32_t t = sp.start + (r - sp.row0);
+    const float* xr = p.x + (size_t)r * p.ldx;
+    const uint32_t kw = p.rank + p.rope_dim, half = p.rope_dim / 2;
+    const float* cs = p.rope_dim ? p.cosines + (size_t)t * p.rope_dim : nullptr;
+    const float* sn = p.rope_dim ? p.sines + (size_t)t * p.rope_dim : nullptr;
+    // pair i of a rotated part: coordinates (2i, 2i + 1) or (i, i + half)
+    auto lo_of = [&](uint32_t i) { return p.interleaved ? 2 * i : i; };
+    auto hi_of = [&](uint32_t i) { return p.interleaved ? 2 * i + 1 : i + half; };
+    if (wave == 0 && p.caches) {
+        const float* c = xr + p.c_col;
+        float ss = 0.0f;
+        for (uint32_t i = lane; i < p.rank; i += 64) ss = fmaf(c[i], c[i], ss);
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)p.rank + p.eps);
+        void* cache = p.caches[q];
+        const size_t base = (size_t)t * kw;
+        for (uint32_t i = lane; i < p.rank; i += 64) {
+            const float v = c[i] * inv * p.scales[i];
+            if (p.cache_bf16) ((uint16_t*)cache)[base + i] = f32_to_bf16(v);
+            else ((float*)cache)[base + i] = v;
+        }
+        const float* kr = c + p.rank;
+        for (uint32_t i = lane; i < half; i += 64) {
+            const float u = kr[lo_of(i)], v = kr[hi_of(i)], co = cs[i], si = sn[i];
+            const float a = u * co - v * si, b = v * co + u * si;
+            if (p.cache_bf16) ((uint16_t*)cache)[base + p.rank + lo_of(i)] = f32_to_bf16(a), ((uint16_t*)cache)[base + p.rank + hi_of(i)] = f32_to_bf16(b);
+            else ((float*)cache)[base + p.rank + lo_of(i)] = a, ((float*)cache)[base + p.rank + hi_of(i)] = b;
+        }
+    }
+    if (!p.qlat) return;
+    for (uint32_t idx = threadIdx.x; idx < p.heads * half; idx += 256) {
+        const uint32_t a = idx / half, i = idx - a * half;
+        const float* qr = xr + (size_t)a * p.q_width + (p.q_width - p.rope_dim);
+        float* dst = p.qlat + ((size_t)r * p.heads + a) * kw + p.rank;
+        const float u = qr[lo_of(i)], v = qr[hi_of(i)], co = cs[i], si = sn[i];
+        dst[lo_of(i)] = u * co - v * si;
+        dst[hi_of(i)] = v * co + u * si;
+    }
+}
+
 // Simple form: a wave per (row, head), lane = latent elements lane, lane + 64, ...; the keys one after the other with a running maximum.
 template <int NT>
 __global__ void __launch_bounds__(256) latent_attention_rows_kernel(LatentAttentionParams p) {
@@ -294,6 +339,14 @@ uzu_status latent_norm_append(hipStream_t s, const float* x, const float* scales
     UZU_REQUIRE(x && scales && caches && spans && row_seq && rank, "latent_norm_append: null argument");
     return launch_check([&] { hipLaunchKernelGGL(latent_norm_append_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, x, scales, eps, caches, cache_bf16, spans, row_seq, rows, rank); },
                         "latent_norm_append");
+}
+
+uzu_status latent_rope_append(hipStream_t s, const LatentRopeAppendParams& p) {
+    if (!p.rows) return UZU_OK;
+    UZU_REQUIRE(p.x && p.spans && p.row_seq && p.rank && (!p.caches || p.scales), "latent_rope_append: null argument");
+    UZU_REQUIRE(p.rope_dim % 2 == 0 && (!p.rope_dim || (p.cosines && p.sines && p.q_width >= p.rope_dim)), "latent_rope_append: an even rotated width with its tables");
+    UZU_REQUIRE(p.c_col + p.rank + p.rope_dim <= p.ldx && (!p.qlat || p.heads * p.q_width <= p.ldx), "latent_rope_append: columns outside the row");
+    return launch_check([&] { hipLaunchKernelGGL(latent_rope_append_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "latent_rope_append");
 }
 
 uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p) {

@@ -124,7 +124,11 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
                 if (p.act == 1) {
                     const float t = fmaxf(v, 0.0f);
                     v = t * t;
+                } else if (p.act == 2) {
+                    v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
                 }
+                if (p.y_scale != 0.0f) v *= p.y_scale;
+                if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)row * p.ldgate + z]));
                 if (p.residual) v += p.residual[(size_t)row * p.ldr + n];
                 y[(size_t)row * p.ldy + n] = v;
             }

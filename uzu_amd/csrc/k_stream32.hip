@@ -47,7 +47,8 @@ __global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tok
 }
 
 // a workgroup per row: the sum of squares as 256 strided partial sums folded in a fixed tree, then the scaled row
-__global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t d) {
+__global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t d,
+                                                            float offset) {
     __shared__ float s_red[256];
     const uint32_t r = blockIdx.x;
     const float* xr = x + (size_t)(row_index ? row_index[r] : r) * d;
@@ -63,8 +64,43 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, floa
     float* o = out + (size_t)r * d;
     for (uint32_t i = threadIdx.x; i < d; i += 256) {
         const float v = xr[i] * inv * gain;
-        o[i] = scales ? v * scales[i] : v;
+        o[i] = scales ? v * (scales[i] + offset) : v;
     }
+}
+
+// the same sum of squares over a sublayer's result y; the normed row joins the stream: out = residual + y * inv * (scales + offset) * layer_scale
+__global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale,
+                                                                float eps, uint32_t d) {
+    __shared__ float s_red[256];
+    const uint32_t r = blockIdx.x;
+    const float* yr = y + (size_t)r * d;
+    float acc = 0.0f;
+    for (uint32_t i = threadIdx.x; i < d; i += 256) acc = fmaf(yr[i], yr[i], acc);
+    s_red[threadIdx.x] = acc;
+    __syncthreads();
+    for (uint32_t w = 128; w > 0; w >>= 1) {
+        if (threadIdx.x < w) s_red[threadIdx.x] += s_red[threadIdx.x + w];
+        __syncthreads();
+    }
+    const float inv = 1.0f / sqrtf(s_red[0] / (float)d + eps);
+    const float* res = residual + (size_t)r * d;
+    float* o = out + (size_t)r * d;
+    for (uint32_t i = threadIdx.x; i < d; i += 256) {
+        float v = yr[i] * inv * (scales[i] + offset);
+        if (layer_scale) v *= layer_scale[i];
+        o[i] = res[i] + v;
+    }
+}
+
+__device__ __forceinline__ float gelu_tanh_f32(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+
+__global__ void __launch_bounds__(256) side_gate_mul_kernel(float* g, const uint32_t* tokens, const uint16_t* table, uint32_t table_ld, uint32_t col0, uint32_t vocab, uint32_t dim) {
+    const uint32_t r = blockIdx.x;
+    uint32_t t = tokens[r];
+    if (t >= vocab) t = 0;
+    const uint16_t* e = table + (size_t)t * table_ld + col0;
+    float* row = g + (size_t)r * dim;
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) row[i] = gelu_tanh_f32(row[i]) * bf16_to_f32(e[i]);
 }
 
 __global__ void __launch_bounds__(256) dyn_tanh_kernel(DynTanhParams p) {
@@ -115,7 +151,19 @@ __device__ __forceinline__ float apply_act(float v, uint32_t act) {
         const float t = fmaxf(v, 0.0f);
         return t * t;
     }
+    if (act == 2) return gelu_tanh_f32(v);
     return v;
+}
+// what follows the activation: the product's scale, a per-(row, product) sigmoid gate
+__device__ __forceinline__ float apply_tail(float v, const LinearF32Params& p, uint32_t r, uint32_t z) {
+    if (p.y_scale != 0.0f) v *= p.y_scale;
+    if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)r * p.ldgate + z]));
+    return v;
+}
+
+__global__ void __launch_bounds__(256) gated_act_rows_kernel(const float* y1, float* hidden, uint32_t ff, ExpertAct act) {
+    const float* src = y1 + (size_t)blockIdx.x * 2 * ff;
+    for (uint32_t f = threadIdx.x; f < ff; f += blockDim.x) hidden[(size_t)blockIdx.x * ff + f] = expert_act(src[ff + f], src[f], act);
 }
 
 // ---- few rows: a wave per output column, RT rows per pass over the weights
@@ -166,7 +214,7 @@ __global__ void __launch_bounds__(256) linear_rows_kernel(LinearF32Params p, uin
         for (int i = 0; i < RT; ++i) {
             const uint32_t r = r0 + i;
             if (r >= p.rows) break;
-            float v = apply_act(acc[i] + bias, p.act);
+            float v = apply_tail(apply_act(acc[i] + bias, p.act), p, r, z);
             if (p.residual) v += p.residual[(size_t)r * p.ldr + n];
             y[(size_t)r * p.ldy + n] = v;
         }
@@ -221,7 +269,7 @@ __global__ void __launch_bounds__(256) linear_tile_kernel(LinearF32Params p) {
         for (int j = 0; j < 4; ++j) {
             const uint32_t n = n0 + tx * 4 + j;
             if (n >= p.n) continue;
-            float v = apply_act(acc[i][j] + (p.bias ? bf16_to_f32(p.bias[n]) : 0.0f), p.act);
+            float v = apply_tail(apply_act(acc[i][j] + (p.bias ? bf16_to_f32(p.bias[n]) : 0.0f), p.act), p, r, z);
             if (p.residual) v += p.residual[(size_t)r * p.ldr + n];
             y[(size_t)r * p.ldy + n] = v;
         }
@@ -446,10 +494,31 @@ uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t*
     return launch_check([&] { hipLaunchKernelGGL(embed_rows_f32_kernel, dim3(rows), dim3(256), 0, s, tokens, table, out, vocab, d, scale); }, "embed_rows_f32");
 }
 
-uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d) {
+uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d,
+                         float offset) {
     if (!rows) return UZU_OK;
     UZU_REQUIRE(x && out && d, "rms_norm_rows: null argument");
-    return launch_check([&] { hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, s, x, out, scales, gain, eps, row_index, d); }, "rms_norm_rows");
+    return launch_check([&] { hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, s, x, out, scales, gain, eps, row_index, d, offset); }, "rms_norm_rows");
+}
+
+uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
+                             uint32_t rows, uint32_t d) {
+    if (!rows) return UZU_OK;
+    UZU_REQUIRE(y && residual && out && scales && d, "rms_norm_add_rows: null argument");
+    return launch_check([&] { hipLaunchKernelGGL(rms_norm_add_rows_kernel, dim3(rows), dim3(256), 0, s, y, residual, out, scales, offset, layer_scale, eps, d); },
+                        "rms_norm_add_rows");
+}
+
+uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act) {
+    if (!rows || !ff) return UZU_OK;
+    UZU_REQUIRE(y1 && hidden, "gated_act_rows: null argument");
+    return launch_check([&] { hipLaunchKernelGGL(gated_act_rows_kernel, dim3(rows), dim3(256), 0, s, y1, hidden, ff, act); }, "gated_act_rows");
+}
+
+uzu_status side_gate_mul(hipStream_t s, float* g, const uint32_t* tokens, const uint16_t* table, uint32_t table_ld, uint32_t col0, uint32_t vocab, uint32_t rows, uint32_t dim) {
+    if (!rows || !dim) return UZU_OK;
+    UZU_REQUIRE(g && tokens && table && col0 + dim <= table_ld, "side_gate_mul: null argument or a slice outside the table's rows");
+    return launch_check([&] { hipLaunchKernelGGL(side_gate_mul_kernel, dim3(rows), dim3(dim < 256 ? 64 : 256), 0, s, g, tokens, table, table_ld, col0, vocab, dim); }, "side_gate_mul");
 }
 
 uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p) {

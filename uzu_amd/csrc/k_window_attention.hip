@@ -28,6 +28,21 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeAppendParams p) {
     const uint32_t half = p.rope_dim / 2;
     const float* cs = p.cosines + (size_t)t * p.rope_dim;
     const float* sn = p.sines + (size_t)t * p.rope_dim;
+    if (p.q_norm || p.k_norm) { // a wave per head: x <- x / sqrt(mean(x^2) + eps) * w over the head's coordinates, in front of the rotation
+        const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        for (uint32_t a = wave; a < p.heads + p.kv_heads; a += 4) {
+            const bool is_q = a < p.heads;
+            const float* w = is_q ? p.q_norm : p.k_norm;
+            if (!w) continue;
+            float* h = is_q ? row + (size_t)a * p.dim : row + p.k_col + (size_t)(a - p.heads) * p.dim;
+            float ss = 0.0f;
+            for (uint32_t i = lane; i < p.dim; i += 64) ss = fmaf(h[i], h[i], ss);
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float)p.dim + p.norm_eps);
+            for (uint32_t i = lane; i < p.dim; i += 64) h[i] = h[i] * inv * w[i];
+        }
+        __syncthreads();
+    }
     for (uint32_t idx = threadIdx.x; idx < p.heads * half; idx += 256) {
         const uint32_t a = idx / half, i = idx - a * half;
         float* h = row + (size_t)a * p.dim;

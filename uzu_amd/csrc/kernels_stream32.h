@@ -6,6 +6,7 @@
 //   k_latent_attention.hip   latent normalisation + cache append, the latent-space attention core (prompt rows and decode rows)
 //   k_window_attention.hip   rotation + key / value cache append, attention over cached keys and values (grouped heads, score cap, window, sinks)
 //   k_retention.hip          retention: the decayed outer-product state (token by token and in chunks), per-head RMS division + gate
+//   k_gated_lru.hip          the gated linear recurrent unit: short causal convolution over a carried window, gates / decays / state update
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -25,8 +26,15 @@ struct SeqSpan {
 uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t* table, float* out, uint32_t rows, uint32_t vocab, uint32_t d, float scale = 1.0f);
 
 // RMS norm with one gain: out[r, :] = gain * x[src(r), :] / sqrt(mean(x[src(r), :]^2) + eps),   src(r) = row_index ? row_index[r] : r.
-// scales (f32 [d], optional) multiplies per coordinate on top.  The row's sum of squares is taken in a fixed order.
-uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d);
+// scales (f32 [d], optional) multiplies per coordinate on top, as (scales[i] + offset): a weight stored around zero has offset 1.  The row's sum of squares is
+// taken in a fixed order.
+uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d,
+                         float offset = 0.0f);
+
+// A sublayer's result joins the stream behind its own norm:  out[r, :] = residual[r, :] + y[r, :] / sqrt(mean(y[r, :]^2) + eps) * (scales + offset) * layer_scale
+// (scales f32 [d]; layer_scale f32 [d] or null; out may alias residual).  The same fixed-order sum of squares as rms_norm_rows.
+uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
+                             uint32_t rows, uint32_t d);
 
 // Dynamic-tanh norm, optionally followed by the token shift:
 //   h[r]   = tanh(alpha * x[src(r)]) * scales + biases          src(r) = row_index ? row_index[r] : r
@@ -53,7 +61,7 @@ uzu_status depth_mix(hipStream_t s, const float* slots, size_t slot_stride, cons
 
 // Y[z][r, n] = act(sum_k X[z][r, k] * W[z][n, k] + bias[n]) + residual[r, n]        z < batch (grid.z): a batch of independent products of one shape
 //   X[z] = x + z * x_batch (row pitch ldx), W[z] = w + z * w_batch ([n, k] bf16), Y[z] = y + z * y_batch (row pitch ldy)
-//   act: 0 none, 1 max(.,0)^2.  residual (pitch ldr, only with batch == 1) may alias y.
+//   act: 0 none, 1 max(.,0)^2, 2 gelu (tanh form).  residual (pitch ldr, only with batch == 1) may alias y.
 struct LinearF32Params {
     const float* x;
     const uint16_t* w;
@@ -66,6 +74,9 @@ struct LinearF32Params {
     size_t x_batch, w_batch, y_batch; // element strides
     uint32_t act;
     uint32_t bf16_products;
+    float y_scale;     // != 0: the product (behind bias and act, before the residual) is multiplied by it
+    const float* gate; // batched products: product z of row r is multiplied by sigmoid(gate[r * ldgate + z]) (a scalar gate per head); null = none
+    uint32_t ldgate;
     // Grouped form (matrix-core kernel only; the experts of a mixture, each with its own bucket of rows): product z covers rows row_offsets[z] ..
     // row_offsets[z + 1] - 1 of X and Y (device array [batch + 1]; x_batch / y_batch unused, `rows` = an upper bound of the total for the grid).
     const uint32_t* row_offsets;
@@ -91,6 +102,11 @@ uzu_status moe_route_topk(hipStream_t s, const float* x, const uint16_t* router,
 struct ExpertAct {
     float alpha = 1.0f, gate_min = -INFINITY, gate_max = INFINITY, up_min = -INFINITY, up_max = INFINITY, up_offset = 0.0f;
 };
+// The gated product of a dense block: hidden[r, f] = act(gate = y1[r, ff + f], up = y1[r, f])   (y1 f32 [rows][2 ff]: up rows first, as the packed projection yields them)
+uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act);
+// Per-layer token input: g[r, j] <- gelu_tanh(g[r, j]) * f32(table[token[r], col0 + j])   (g f32 [rows][dim]; table bf16 [vocab][table_ld]; an id >= vocab reads row 0)
+uzu_status side_gate_mul(hipStream_t s, float* g, const uint32_t* tokens, const uint16_t* table, uint32_t table_ld, uint32_t col0, uint32_t vocab, uint32_t rows, uint32_t dim);
+
 // hidden[r * top + j, f] = act(gate_e x_r, up_e x_r) for e = ids[r, j] < routed; w13 bf16 [routed][2 ff][d], rows [0, ff) of an expert = up, [ff, 2 ff) = gate
 uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,
                                uint32_t top, uint32_t bf16_products, const ExpertAct& act = ExpertAct());
@@ -148,6 +164,30 @@ bool latent_attention_tiled_supported(const LatentAttentionParams& p);
 uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p);
 constexpr uint32_t kLatentMaxRank = 2048;
 
+// What stands between the packed projection and the latent-space core when the cache row carries a rotated key part: row r of `x` (f32, pitch ldx) holds the down
+// projection's rank + rope_dim numbers at column c_col and the queries [heads][q_width] at column 0, the last rope_dim coordinates of a query head being its
+// rotated part.  The latent (first rank numbers) is RMS-normed with `scales`; the rope_dim numbers behind it turn by the row's position (tables f32
+// [positions][rope_dim] as rope_append reads them; interleaved: pairs (2i, 2i + 1), else (i, i + rope_dim / 2)) and are NOT normed; [latent | rotated part] goes to
+// row t of the sequence's cache (width rank + rope_dim, bf16 or f32).  Every query head's rotated part turns the same way and lands in
+// qlat[r, head, rank .. rank + rope_dim) (qlat f32 [rows][heads][rank + rope_dim]; the first rank columns of a head are filled by the folded key projection).
+// rope_dim == 0: normalisation + append alone.
+struct LatentRopeAppendParams {
+    const float* x;
+    uint32_t ldx, c_col, rank, rope_dim;
+    const float* scales;
+    float eps;
+    void* const* caches;
+    uint32_t cache_bf16;
+    uint32_t heads, q_width;
+    float* qlat;
+    const float *cosines, *sines;
+    uint32_t interleaved;
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t rows;
+};
+uzu_status latent_rope_append(hipStream_t s, const LatentRopeAppendParams& p);
+
 // Rotation of queries and keys, key scaling, and the append of keys and values to the sequences' caches -- what stands between the packed projection and the
 // mixer's core.  Row r of `qkv` (f32, pitch ld) holds queries [heads][dim] at column 0, keys [kv_heads][dim] at column k_col and values [kv_heads][vdim] at
 // column v_col.  The first rope_dim coordinates of every query and key head turn by the angle of the row's position t: with half = rope_dim / 2,
@@ -155,12 +195,15 @@ constexpr uint32_t kLatentMaxRank = 2048;
 // and keys are multiplied by key_scale afterwards.  Queries are replaced in place.  With caches (key_caches / value_caches: device arrays [nseq] of pointers to
 // [positions][kv_heads * dim] and [positions][kv_heads * vdim], bf16 or f32) rotated keys and values go to row t of the sequence's caches; without (null) the
 // keys are replaced in place and values stay where they are.  kv_heads == 0: the row carries queries only (a layer that reads another layer's cache).
+// q_norm / k_norm (f32 [dim], optional): every query / key head is RMS-normed over its dim coordinates (norm_eps, plain weights) in front of the rotation.
 struct RopeAppendParams {
     float* qkv;
     uint32_t ld, k_col, v_col;
     uint32_t heads, kv_heads, dim, vdim, rope_dim;
     const float *cosines, *sines;
     float key_scale;
+    const float *q_norm, *k_norm;
+    float norm_eps;
     void* const* key_caches;
     void* const* value_caches;
     uint32_t cache_bf16;
@@ -227,6 +270,34 @@ uzu_status retention(hipStream_t s, const RetentionParams& p);
 // Per head: x[r, a, :] <- x[r, a, :] / sqrt(mean(x[r, a, :]^2) + eps) * silu(gate[r, a * width ...])   (x f32 [rows][heads * width] in place; gate f32 rows of
 // pitch ldg; gate == null: the division alone)
 uzu_status head_rms_gate(hipStream_t s, float* x, const float* gate, uint32_t ldg, float eps, uint32_t rows, uint32_t heads, uint32_t width);
+
+// Gated linear recurrent unit behind a short causal convolution (k_gated_lru.hip).  Row r (sequence z, position t) of `branches` (f32, pitch ld) holds the gate
+// branch's `width` numbers at column 0 and the recurrent branch's at column x_col.
+//   lru_conv:  u[r, c] = conv_b[c] + sum_j conv_w[c, j] * xin(t - (taps - 1) + j, c)     xin = the recurrent branch of the sequence's earlier rows: of this pass, or
+//              (in front of the pass) the taps - 1 inputs the state keeps ([taps - 1][width] f32, oldest first), or zero in front of position 0.  u f32 [rows][width].
+//   lru_scan:  with g = the gate pre-activations [rows][blocks][2 bw] (recurrence gate's bw numbers, then the input gate's) and their biases,
+//              a = exp(-rate * sigmoid(g_r + b_r) * softplus(lambda)),  S <- a S + sqrt(1 - a^2) * sigmoid(g_i + b_i) * u,  out[r, c] = S * gelu_tanh(gate branch);
+//              S starts from the sequence's state (zero at position 0) and is left there behind the pass's last row, and so are the last taps - 1 inputs.
+//              All f32.  form 0: chosen by the row count; 1: position by position; 2: in pieces of a sequence's rows, each scanned from zero with its decay product,
+//              the pieces' carries joined in order (differs from form 1 by f32 rounding only).
+struct GatedLruParams {
+    const float* branches;
+    uint32_t ld, x_col;
+    float* u;            // [rows][width]
+    const float* gates;  // [rows][2 width]
+    float* out;          // [rows][width]
+    const float *conv_w, *conv_b, *gate_b, *lambda;
+    float rate;
+    float* const* states;      // device array [nseq]: f32 [width]
+    float* const* conv_states; // device array [nseq]: f32 [taps - 1][width]
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t nseq, rows, width, blocks, taps;
+    uint32_t form;
+    uint32_t max_count; // the longest sequence share of the pass (the caller knows the counts)
+};
+uzu_status lru_conv(hipStream_t s, const GatedLruParams& p);
+uzu_status lru_scan(hipStream_t s, const GatedLruParams& p);
 
 } // namespace k
 } // namespace uzu

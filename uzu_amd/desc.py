@@ -18,7 +18,7 @@ import numpy as np
 # enums (uzu_model_desc.h)
 QUANT_SCALE_BIAS, QUANT_SCALE_ZERO_POINT, QUANT_SCALE_SYMMETRIC, QUANT_NONE = 0, 1, 2, 3
 ACT_SILU, ACT_GELU_APPROX, ACT_GELU_EXACT, ACT_IDENTITY, ACT_SOFTPLUS, ACT_RELU_SQUARED = 0, 1, 2, 3, 4, 5
-MIXER_ATTENTION, MIXER_DELTA_NET, MIXER_LATENT_ATTENTION, MIXER_RETENTION = 0, 1, 2, 3
+MIXER_ATTENTION, MIXER_DELTA_NET, MIXER_LATENT_ATTENTION, MIXER_RETENTION, MIXER_GATED_LRU = 0, 1, 2, 3, 4
 NORM_STATISTICS, NORM_DYNAMIC_TANH, NORM_RMS_SCALAR = 0, 1, 2
 MOE_ROUTE_TOPK_LOGITS, MOE_ROUTE_SCORES = 0, 1
 ROPE_NONE, ROPE_UNSCALED, ROPE_LLAMA, ROPE_LINEAR, ROPE_YARN, ROPE_LONGROPE = 0, 1, 2, 3, 4, 5
@@ -98,7 +98,12 @@ class LayerDesc(C.Structure):
         ("token_shift", C.c_void_p), ("depth_weights", C.c_void_p),
         ("num_depth_weights", C.c_uint32), ("mlp_plain", C.c_uint32), ("no_mlp", C.c_uint32), ("parallel_block", C.c_uint32),
         ("score_soft_cap", C.c_float), ("unit_sink", C.c_uint32), ("key_scale", C.c_float), ("head_norm_epsilon", C.c_float),
-        ("retention_decay", C.c_void_p), ("reserved4", C.c_uint32), ("reserved6", C.c_uint32),
+        ("retention_decay", C.c_void_p),
+        ("latent_rope_dim", C.c_uint32), ("latent_packed", C.c_uint32), ("rope_interleaved", C.c_uint32),
+        ("lru_width", C.c_uint32), ("lru_blocks", C.c_uint32), ("lru_decay_rate", C.c_float),
+        ("lru_gate_weights", C.c_void_p), ("lru_gate_biases", C.c_void_p), ("lru_lambda", C.c_void_p),
+        ("layer_scale_mixer", C.c_void_p), ("layer_scale_mlp", C.c_void_p),
+        ("ple_slice", C.c_uint32), ("weights_of_layer", C.c_uint32), ("stream_reentry", LinearDesc),
     ]
 
 
@@ -317,6 +322,33 @@ class LayerWeights:
     key_scale: float = 0.0
     head_norm_epsilon: float = 0.0
     retention_decay: Optional[np.ndarray] = None  # f32 [num_heads]
+    # f32-stream designs: latent attention with a rotated key part shared by the heads (the cache row is [latent | rotated part]), its down projection and a
+    # per-head sigmoid gate (has_gate) packed behind the queries; rotation in interleaved pairs
+    latent_rope_dim: int = 0
+    latent_packed: bool = False
+    rope_interleaved: bool = False
+    # gated linear recurrent unit (mixer_kind MIXER_GATED_LRU): qkv_projection rows = gate branch | recurrent branch (with biases); the short convolution uses
+    # dn_kernel_size / dn_conv_weights / dn_conv_biases; block-diagonal gates
+    lru_width: int = 0
+    lru_blocks: int = 0
+    lru_decay_rate: float = 0.0
+    lru_gate_weights: Optional[np.ndarray] = None  # bf16 bits [blocks][2 bw][bw]: the recurrence gate's rows, then the input gate's
+    lru_gate_biases: Optional[np.ndarray] = None   # f32 [blocks][2 bw]
+    lru_lambda: Optional[np.ndarray] = None        # f32 [lru_width]
+    layer_scale_mixer: Optional[np.ndarray] = None  # f32 [model_dim]: on the mixer's (post-normed) result
+    layer_scale_mlp: Optional[np.ndarray] = None
+    gated_act: Optional[tuple] = None              # a gated dense MLP's (slope, (gate_min, gate_max), (up_min, up_max), up_offset) in an f32-stream design
+    ple_slice: int = 0                             # which ple_dim-wide slice of the side table's row this layer run reads
+    weights_of_layer: Optional[int] = None         # this run uses the tensors of that earlier run (a looped stack); its state is its own
+    stream_reentry: Optional[LinearWeights] = None  # x <- W [x ; x0] in front of this run, [model_dim, 2 model_dim]
+
+    def _moe_desc(self) -> MoeDesc:
+        if self.moe is not None:
+            return self.moe.desc()
+        if self.gated_act is not None:
+            slope, gate, up, off = self.gated_act
+            return MoeDesc(0, 0, 0, 0, 2, float(slope), float(gate[0]), float(gate[1]), float(up[0]), float(up[1]), None, None, None, None, None, None, 0, 0, None, float(off), 0)
+        return MoeDesc()
 
     def desc(self) -> LayerDesc:
         empty = LinearDesc()
@@ -341,15 +373,18 @@ class LayerWeights:
             int(self.ple is not None), self.ple.ple_dim if self.ple else 0, self.ple.activation if self.ple else 0, int(self.is_non_causal),
             ld(self.ple.gate if self.ple else None), ld(self.ple.projection if self.ple else None),
             (self.ple.norm if self.ple else ABSENT_NORM).desc(),
-            self.moe.desc() if self.moe is not None else MoeDesc(),
+            self._moe_desc(),
             int(self.latent_rank), int(self.value_head_dim), ld(self.latent_down), self.latent_norm.desc(), ld(self.latent_up_keys), ld(self.latent_up_values),
             _ptr(self.token_shift), _ptr(self.depth_weights), 0 if self.depth_weights is None else int(self.depth_weights.size), int(self.mlp_plain), int(self.no_mlp), int(self.parallel_block),
-            float(self.score_soft_cap), int(self.unit_sink), float(self.key_scale), float(self.head_norm_epsilon), _ptr(self.retention_decay), 0, 0,
+            float(self.score_soft_cap), int(self.unit_sink), float(self.key_scale), float(self.head_norm_epsilon), _ptr(self.retention_decay),
+            int(self.latent_rope_dim), int(self.latent_packed), int(self.rope_interleaved), int(self.lru_width), int(self.lru_blocks), float(self.lru_decay_rate),
+            _ptr(self.lru_gate_weights), _ptr(self.lru_gate_biases), _ptr(self.lru_lambda), _ptr(self.layer_scale_mixer), _ptr(self.layer_scale_mlp),
+            int(self.ple_slice), 0 if self.weights_of_layer is None else int(self.weights_of_layer) + 1, ld(self.stream_reentry),
         )
 
     def linears(self):
         names = ("qkv_projection", "gate_projection", "out_projection", "dn_in_proj", "dn_out_proj", "up_projection",
-                 "down_projection", "latent_down", "latent_up_keys", "latent_up_values")
+                 "down_projection", "latent_down", "latent_up_keys", "latent_up_values", "stream_reentry")
         out = [(n, getattr(self, n)) for n in names if getattr(self, n) is not None]
         if self.ple is not None:
             out += [("ple.gate", self.ple.gate), ("ple.projection", self.ple.projection)]
@@ -510,6 +545,8 @@ class ModelBundle:
     ple: Optional[PleModelWeights] = None
     f32_stream: bool = False                     # an f32-stream design (include/uzu_model_desc.h): its own forward encoder, f32 logits, batched steps
     architecture: Optional[str] = None           # config.json `architecture` of a design that is not in the reference's config schema
+    side_table: Optional[LinearWeights] = None   # f32-stream designs: a second token table [vocab, slices * side_dim]; a layer with `ple` reads its slice of the token's row
+    side_dim: int = 0
     _keep: list = field(default_factory=list, repr=False)
 
     def desc(self) -> ModelDesc:
@@ -522,6 +559,11 @@ class ModelBundle:
             self._keep.append(ropes)
         e = LinearDesc()
         p = self.ple
+        if p is None and self.side_table is not None:  # the side table alone: no model projection, no projection norm
+            return ModelDesc(self.vocab_size, self.model_dim, len(self.layers), int(self.tied_embeddings), self.input_scale, self.logit_scale, self.logit_soft_cap,
+                             self.max_context_length, self.rope.desc(), self.embedding.desc(), out_emb, self.output_norm.desc(), C.cast(arr, C.POINTER(LayerDesc)),
+                             len(self.ropes) if self.ropes else 0, 1, C.cast(ropes, C.POINTER(RopeDesc)) if ropes is not None else None, self.embedding_norm.desc(),
+                             int(self.side_dim), int(self.side_table.n), 1.0, 0.0, 0.0, 0, self.side_table.desc(), e, ABSENT_NORM.desc(), int(self.f32_stream), 0)
         return ModelDesc(self.vocab_size, self.model_dim, len(self.layers), int(self.tied_embeddings),
                          self.input_scale, self.logit_scale, self.logit_soft_cap, self.max_context_length,
                          self.rope.desc(), self.embedding.desc(), out_emb, self.output_norm.desc(),
@@ -537,7 +579,7 @@ class ModelBundle:
     # ---- algorithmic bytes per decoded token (SURVEY.md §8d formula) ----
     def weight_stream_bytes(self) -> int:
         total = 0
-        for l in self.layers:
+        for l in self.layers:  # (a run that shares an earlier run's tensors streams them again)
             for _, w in l.linears():
                 total += w.nbytes()
             if l.moe is not None:
@@ -558,7 +600,10 @@ class ModelBundle:
                 total += 2 * l.num_heads * l.head_dim * l.value_head_dim * 4  # f32 state read + write
             elif l.mixer_kind == MIXER_LATENT_ATTENTION:
                 rows = min(context, l.sliding_window_size) if l.sliding_window_size else context
-                total += rows * l.latent_rank * 2                             # one latent row per visible token, bf16, shared by all heads
+                total += rows * (l.latent_rank + l.latent_rope_dim) * 2       # one latent row (+ the shared rotated key part) per visible token, bf16
+            elif l.mixer_kind == MIXER_GATED_LRU:
+                total += 2 * l.lru_width * l.dn_kernel_size * 4               # f32 state + the convolution's inputs, read + write
+                total += 2 * l.lru_width * (l.lru_width // max(l.lru_blocks, 1)) * 2  # the block-diagonal gate matrices, bf16
             else:
                 total += 2 * l.dn_num_heads * l.dn_value_head_dim * l.dn_head_dim * 4  # f32 state read + write
                 conv_dim = 2 * l.dn_num_groups * l.dn_head_dim + l.dn_num_heads * l.dn_value_head_dim
@@ -592,7 +637,9 @@ class ModelBundle:
             elif l.mixer_kind == MIXER_LATENT_ATTENTION:  # scores and weighted sum in latent space, over the window
                 w = l.sliding_window_size
                 vis = pairs if not w else min(pairs, tokens * float(w))
-                flops += 4.0 * vis * l.num_heads * l.latent_rank
+                flops += 4.0 * vis * l.num_heads * l.latent_rank + 2.0 * vis * l.num_heads * l.latent_rope_dim
+            elif l.mixer_kind == MIXER_GATED_LRU:  # the two block-diagonal gate products; convolution and recurrence are element-wise
+                flops += 4.0 * tokens * l.lru_width * (l.lru_width // max(l.lru_blocks, 1))
             else:  # delta rule: ~6 flops per state element per token (decay, S k, rank-1 update, S q)
                 flops += 6.0 * tokens * l.dn_num_heads * l.dn_value_head_dim * l.dn_head_dim
         return flops

@@ -1,4 +1,4 @@
-"""What the readers of designs with their own ``config.json`` schema (uzu_amd.lazolix, uzu_amd.relulix) share: bf16 tensors of a safetensors file by name with
+"""What the readers of designs with their own ``config.json`` schema (uzu_amd.lazolix, uzu_amd.relulix, uzu_amd.begasun) share: bf16 tensors of a safetensors file by name with
 shape checks, bf16 bit patterns, and a full-precision linear of the engine's description."""
 from __future__ import annotations
 

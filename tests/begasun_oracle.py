@@ -222,3 +222,139 @@ def forward(cfg: dict, W: Dict[str, np.ndarray], tokens) -> Tuple[np.ndarray, np
         taps.append(x)
     out = norm_one_plus(x, W["final.norm"], eps)
     return out @ f64(W["head"]).T * float(cfg.get("logit_scale", 1.0)), np.stack(taps)
+
+
+# ---------------------------------------------------------------------------------------------- configurations, random weights and files of the tests' own making
+def rot(dims, base=10000.0, scaling=None):
+    r = {"dims": int(dims), "base": float(base)}
+    if scaling:
+        r["scaling"] = dict(scaling)
+    return r
+
+
+def dense(ff, limit=7.0):
+    return {"kind": "dense", "ff": int(ff), "limit": float(limit)}
+
+
+def latent_layer(heads, dim, rot_dim, vdim, kv_rank, rotation, scale=None, mlp=None):
+    return {"type": "latent_attention", "mlp": mlp, "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "rot": rotation,
+                                                              "scale": float(scale if scale is not None else (dim + rot_dim) ** -0.5)}}
+
+
+def attention_layer(heads, kv_heads, dim, vdim, rotation, scale=None, mlp=None):
+    return {"type": "attention", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot": rotation,
+                                                       "scale": float(scale if scale is not None else dim ** -0.5)}}
+
+
+def rglru_layer(width, blocks, conv, mlp=None):
+    return {"type": "rglru", "mlp": mlp, "mixer": {"width": int(width), "blocks": int(blocks), "conv": int(conv)}}
+
+
+def config(vocab, width, layers, eps=1e-6, embed_scale=None, logit_scale=1.0, loop=None, side_dim=0):
+    cfg = {"architecture": "Begasun", "vocab": int(vocab), "width": int(width), "norm": {"eps": float(eps)},
+           "embedding": {"scale": float(embed_scale if embed_scale is not None else width ** 0.5)}, "layers": layers, "logit_scale": float(logit_scale)}
+    if loop:
+        cfg["loop"] = {"start": int(loop[0]), "stop": int(loop[1]), "times": int(loop[2])}
+    if side_dim:
+        cfg["token_side"] = {"dim": int(side_dim)}
+    return cfg
+
+
+def bf16_bits(a):
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def to_bf16(a):
+    return (bf16_bits(a).astype(np.uint32) << 16).view(np.float32).reshape(np.shape(a))
+
+
+def weights(cfg, seed, logit_gain=1.0):
+    """bf16-representable float32 tensors of every name the configuration implies"""
+    rng = np.random.default_rng(seed)
+    d, V = cfg["width"], cfg["vocab"]
+    W = {}
+
+    def lin(name, n, k, gain=1.0, bias=False):
+        W[name] = to_bf16(rng.standard_normal((n, k)) * gain / np.sqrt(k))
+        if bias:
+            W[name + ".b"] = to_bf16(rng.standard_normal(n) * 0.2)
+
+    def vec(name, n, centre, spread):
+        W[name] = to_bf16(centre + spread * (rng.random(n) - 0.5))
+
+    W["embed"] = to_bf16(rng.standard_normal((V, d)) / cfg["embedding"]["scale"])
+    if cfg.get("loop"):
+        lin("loop.in", d, 2 * d, gain=1.4)
+    side = cfg.get("token_side")
+    if side:
+        W["side.embed"] = to_bf16(rng.standard_normal((V, len(cfg["layers"]) * side["dim"])))
+    for i, lc in enumerate(cfg["layers"]):
+        p, mx = f"l{i}.", lc["mixer"]
+        vec(p + "norm1", d, 0.0, 0.4), vec(p + "norm1b", d, 0.0, 0.4), vec(p + "ls1", d, 0.8, 0.8)
+        if lc["type"] == "latent_attention":
+            H, dim, rd, vd, rank = mx["heads"], mx["dim"], mx["rot_dim"], mx["vdim"], mx["kv_rank"]
+            lin(p + "mix.q", H * (dim + rd), d, 2.5), lin(p + "mix.dkv", rank + rd, d, 2.5), lin(p + "mix.g", H, d, 2.0)
+            vec(p + "mix.dkv.norm", rank, 1.0, 0.6)
+            lin(p + "mix.uk", H * dim, rank, 1.5), lin(p + "mix.uv", H * vd, rank), lin(p + "mix.o", d, H * vd)
+        elif lc["type"] == "attention":
+            H, G, dim, vd = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+            lin(p + "mix.q", H * dim, d, 2.0), lin(p + "mix.k", G * dim, d, 2.0), lin(p + "mix.v", G * vd, d)
+            vec(p + "mix.q.norm", dim, 1.6, 0.8), vec(p + "mix.k.norm", dim, 1.6, 0.8)
+            lin(p + "mix.o", d, H * vd)
+        else:
+            w, blocks, taps = mx["width"], mx["blocks"], mx["conv"]
+            bw = w // blocks
+            lin(p + "mix.y", w, d, 1.5, bias=True), lin(p + "mix.x", w, d, 1.5, bias=True)
+            W[p + "mix.conv"] = to_bf16(rng.standard_normal((w, taps)) * 0.6)
+            W[p + "mix.conv.b"] = to_bf16(rng.standard_normal(w) * 0.1)
+            for g in ("ra", "ri"):
+                W[p + "mix." + g] = to_bf16(rng.standard_normal((blocks, bw, bw)) * 1.5 / np.sqrt(bw))
+                W[p + "mix." + g + ".b"] = to_bf16(rng.standard_normal((blocks, bw)) * 0.3)
+            vec(p + "mix.lam", w, -3.0, 4.0)   # decays from about 0.3 up to 0.99 per position
+            lin(p + "mix.o", d, w)
+        if lc.get("mlp") is not None:
+            ff = lc["mlp"]["ff"]
+            vec(p + "norm2", d, 0.0, 0.4), vec(p + "norm2b", d, 0.0, 0.4), vec(p + "ls2", d, 0.8, 0.8)
+            lin(p + "mlp.gate", ff, d, 1.5), lin(p + "mlp.up", ff, d, 1.5), lin(p + "mlp.down", d, ff)
+        if side:
+            lin(p + "side.gate", side["dim"], d, 1.5), lin(p + "side.proj", d, side["dim"])
+            vec(p + "side.norm", d, 0.5, 0.6)
+    vec("final.norm", d, 0.0, 0.4)
+    lin("head", V, d, logit_gain)
+    return W
+
+
+def write_model_dir(path, cfg, W):
+    """config.json + model.safetensors (bf16) in the design's layout, written with nothing but the file format"""
+    import json
+    import os
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(cfg, f)
+    header, blobs, off = {}, [], 0
+    for name in sorted(W):
+        b = bf16_bits(W[name]).tobytes()
+        header[name] = {"dtype": "BF16", "shape": list(np.shape(W[name])), "data_offsets": [off, off + len(b)]}
+        blobs.append(b)
+        off += len(b)
+    hj = json.dumps(header).encode()
+    hj += b" " * (-len(hj) % 8)
+    with open(os.path.join(path, "model.safetensors"), "wb") as f:
+        f.write(len(hj).to_bytes(8, "little") + hj + b"".join(blobs))
+
+
+def logit_error(got, want):
+    """per row: RMS over the vocabulary of the difference with its mean taken off, relative to the RMS of the centred expected row"""
+    d = f64(got) - f64(want)
+    d = d - d.mean(-1, keepdims=True)
+    w = f64(want) - f64(want).mean(-1, keepdims=True)
+    return np.sqrt((d * d).mean(-1)) / np.sqrt((w * w).mean(-1) + 1e-30)
+
+
+def greedy(cfg, W, prompt, n):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        out.append(int(np.argmax(forward(cfg, W, toks)[0][-1])))
+        toks.append(out[-1])
+    return out

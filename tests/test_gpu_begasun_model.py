@@ -1,0 +1,407 @@
+"""Begasun through the engine (HipModel: states, batched steps, prefill / decode, sampling, the generate loops) against the float64 oracle on small models of the
+tests' own making: odd sizes, a loop in front / in the middle / over everything, one to three passes, layers of every type with and without a dense block, one
+and several gate blocks, one and several convolution taps, grouped and single key / value heads, rotated parts narrower than, equal to and wider than the plain
+part, scaled and plain frequencies, with and without the per-layer token input."""
+
+import numpy as np
+import pytest
+
+import begasun_oracle as O
+from uzu_amd import loader
+from uzu_amd.engine import MODEL_BATCH, MODEL_DEBUG_TAPS, MODEL_FULL_F32, HipModel
+
+pytestmark = pytest.mark.gpu
+
+TOL = {True: 4e-5, False: 6e-2}  # full f32 / bf16 products: rms logit error relative to the rms of the logits
+YARN = {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 1.5}
+
+
+def rows_ok(err, full, tol=None):
+    """True f32: every row inside the tolerance.  bf16 products: the rounding noise of a narrow stream grows through the layer runs and a single row can stand out,
+    so nine rows in ten must be inside and the median well inside."""
+    err, tol = np.asarray(err), TOL[full] if tol is None else tol
+    return bool(err.max() < tol) if full else bool(np.median(err) < tol / 2 and np.mean(err < tol) >= 0.9)
+
+
+def cfg_a():  # odd sizes: nothing is a multiple of 8, so every kernel runs its general form; the loop sits behind the first layer and runs three times
+    return O.config(vocab=61, width=36, eps=1e-5, embed_scale=3.5, logit_scale=0.7, side_dim=5, loop=(1, 3, 3), layers=[
+        O.rglru_layer(20, 4, 3, mlp=O.dense(28, 1.0)),
+        O.latent_layer(3, 6, 4, 10, 12, O.rot(4, 5000.0, YARN), scale=0.4, mlp=None),
+        O.attention_layer(6, 2, 10, 6, O.rot(4, 10000.0), scale=0.3, mlp=O.dense(20, 0.7)),
+        O.latent_layer(2, 8, 2, 4, 15, O.rot(2, 100.0), mlp=O.dense(12, 50.0)),
+    ])
+
+
+def cfg_b():  # matrix-core friendly sizes; the loop covers the middle; a recurrent layer with ONE gate block and ONE tap; no token input
+    return O.config(vocab=97, width=64, loop=(1, 4, 2), layers=[
+        O.attention_layer(4, 2, 16, 16, O.rot(8, 10000.0, {"factor": 3.0, "original": 64, "fast": 24.0, "slow": 2.0}), mlp=O.dense(32, 1.75)),
+        O.rglru_layer(64, 2, 4, mlp=None),
+        O.latent_layer(4, 16, 8, 16, 24, O.rot(8, 50000.0, {"factor": 2.0, "original": 64, "fast": 16.0, "slow": 1.0}), mlp=O.dense(48, 2.0)),
+        O.rglru_layer(32, 1, 1, mlp=O.dense(16, 1.0)),
+        O.attention_layer(8, 8, 8, 16, O.rot(8, 10000.0), mlp=None),
+    ])
+
+
+@pytest.fixture(scope="module")
+def models(hip_ctx, tmp_path_factory):
+    out = {}
+    for name, cfg, seed in (("a", cfg_a(), 11), ("b", cfg_b(), 12)):
+        W = O.weights(cfg, seed)
+        path = str(tmp_path_factory.mktemp("begasun") / name)
+        O.write_model_dir(path, cfg, W)
+        bundle = loader.load_model_dir(path, max_context_length=512)
+        W64 = {k: v.astype(np.float64) for k, v in W.items()}
+        out[name] = (cfg, W64, {full: HipModel(hip_ctx, bundle, MODEL_BATCH(6) | MODEL_DEBUG_TAPS | (MODEL_FULL_F32 if full else 0)) for full in (True, False)})
+    yield out
+    for _, _, ms in out.values():
+        for m in ms.values():
+            m.close()
+
+
+def prompt(cfg, n, seed):
+    return list(np.random.default_rng(seed).integers(0, cfg["vocab"], size=n))
+
+
+def make(hip_ctx, tmp_path, cfg, seed, flags=MODEL_FULL_F32, ctx_len=256, edit=None, name="m"):
+    W = O.weights(cfg, seed)
+    if edit:
+        edit(W)
+    O.write_model_dir(str(tmp_path / name), cfg, W)
+    W64 = {k: v.astype(np.float64) for k, v in W.items()}
+    return W64, HipModel(hip_ctx, loader.load_model_dir(str(tmp_path / name), max_context_length=ctx_len), MODEL_BATCH(2) | MODEL_DEBUG_TAPS | flags)
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("full", [True, False])
+def test_whole_prompt_every_position_and_every_layer_run(models, name, full):
+    cfg, W, ms = models[name]
+    m = ms[full]
+    toks = prompt(cfg, 150, 1)  # positions on both sides of the 32-, 64- and 128-key block borders of the attention kernels
+    want, runs = O.forward(cfg, W, toks)
+    st = m.new_state()
+    got, _ = m.step_batch([st], [toks], [list(range(len(toks)))])
+    assert len(runs) == len(O.layer_order(cfg))
+    for l, ref in enumerate(runs):  # the residual stream behind every layer run: names the first run that differs
+        err = np.abs(m.read_layer_output_f32(l) - ref).max(-1) / np.abs(ref).max()
+        assert rows_ok(err, full, 2e-5 if full else 5e-2), (l, err.max(), np.median(err))
+    assert rows_ok(O.logit_error(got, want), full)
+    st.close()
+
+
+def one_layer(layer, vocab=53, width=40, **kw):
+    return O.config(vocab=vocab, width=width, layers=[layer], **kw)
+
+
+MECHANISMS = {
+    "recurrent_unit": one_layer(O.rglru_layer(24, 3, 4)),
+    "recurrent_unit_one_block_two_taps": one_layer(O.rglru_layer(40, 1, 2)),
+    "recurrent_unit_blocks_of_one_channel": one_layer(O.rglru_layer(7, 7, 5)),
+    "latent_attention": one_layer(O.latent_layer(2, 8, 8, 8, 16, O.rot(8, 1e4))),
+    "latent_attention_scaled_rotation_wide": one_layer(O.latent_layer(3, 4, 12, 6, 20, O.rot(12, 1e4, YARN), scale=0.7)),
+    "latent_attention_one_head": one_layer(O.latent_layer(1, 16, 2, 24, 5, O.rot(2, 10.0))),
+    "attention_plain": one_layer(O.attention_layer(2, 2, 8, 8, O.rot(8, 1e4))),
+    "attention_grouped_partial_rotation": one_layer(O.attention_layer(4, 2, 12, 20, O.rot(6, 1e4), scale=0.9)),
+    "attention_one_kv_head_no_rotation": one_layer(O.attention_layer(3, 1, 16, 8, O.rot(0))),
+    "dense_block_tight_clamp": one_layer(O.attention_layer(1, 1, 8, 8, O.rot(2, 1e4), mlp=O.dense(24, 0.25))),
+    "token_input": one_layer(O.attention_layer(1, 1, 8, 8, O.rot(2, 1e4)), side_dim=9),
+    "loop_of_one_layer_four_passes": one_layer(O.rglru_layer(16, 2, 3, mlp=O.dense(8)), loop=(0, 1, 4), side_dim=3),
+    "scales": one_layer(O.attention_layer(2, 1, 8, 8, O.rot(4, 1e4)), embed_scale=0.3, logit_scale=2.5, eps=1e-2),
+}
+
+
+@pytest.mark.parametrize("which", sorted(MECHANISMS))
+def test_each_mechanism_alone_in_a_one_layer_model(hip_ctx, tmp_path, which):
+    cfg = MECHANISMS[which]
+    W, m = make(hip_ctx, tmp_path, cfg, 5)
+    toks = prompt(cfg, 90, 3)
+    want, runs = O.forward(cfg, W, toks)
+    st = m.new_state()
+    got, _ = m.step_batch([st], [toks], [list(range(len(toks)))])
+    for l, ref in enumerate(runs):
+        assert np.abs(m.read_layer_output_f32(l) - ref).max() < 2e-5 * np.abs(ref).max(), l
+    assert O.logit_error(got, want).max() < TOL[True]
+    st.reset()  # and token by token from a reused state: the decode forms of the same kernels
+    rows = [m.step_batch([st], [[t]], [[0]])[0][0] for t in toks[:40]]
+    assert O.logit_error(np.stack(rows), want[:40]).max() < TOL[True]
+    st.close()
+    m.close()
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("full", [True, False])
+def test_prefill_then_token_by_token_and_portions_down_to_two_tokens(models, name, full):
+    cfg, W, ms = models[name]
+    m = ms[full]
+    toks = prompt(cfg, 120, 2)
+    want, _ = O.forward(cfg, W, toks)
+    for cuts in ([100] + [1] * 20, [1] * 30 + [90], [2, 3, 2, 50, 7, 2, 54], [33, 31, 17, 39], [64, 1, 55], [2] * 5 + [110]):
+        assert sum(cuts) == len(toks)
+        st, rows, at = m.new_state(), [], 0
+        for n in cuts:
+            lg, _ = m.step_batch([st], [toks[at:at + n]], [list(range(n))])
+            rows.append(lg)
+            at += n
+        assert st.context_length == len(toks)
+        # (bf16 products: the odd-sized model is narrow and runs its loop three times: its rounding noise is twice the other model's)
+        assert rows_ok(O.logit_error(np.concatenate(rows), want), full, None if full else TOL[False] * (2 if name == "a" else 1)), cuts
+        st.close()
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_unequal_batch_equals_each_request_alone_and_reused_states(models, name):
+    cfg, W, ms = models[name]
+    m = ms[True]
+    reqs = [prompt(cfg, n, 10 + n) for n in (1, 37, 90, 5, 64)]
+    alone = []
+    for r in reqs:
+        st = m.new_state()
+        first, _ = m.step_batch([st], [r[:-3]] if len(r) > 3 else [r], [[len(r) - 4] if len(r) > 3 else [0]])
+        tail = [m.step_batch([st], [[t]], [[0]])[0] for t in (r[-3:] if len(r) > 3 else [])]
+        alone.append(np.concatenate([first] + tail))
+        st.close()
+    pool = [m.new_state() for _ in reqs]
+    for round_ in range(2):  # the second round reuses the states the first one gave back (reset), in another order: caches and recurrent states of other requests
+        states = pool if round_ == 0 else pool[::-1]
+        heads = [r[:-3] if len(r) > 3 else r for r in reqs]
+        lg, _ = m.step_batch(states, heads, [[len(h) - 1] for h in heads])
+        got = [[lg[i]] for i in range(len(reqs))]
+        for step in range(3):  # decoded together; the one-token request has left the batch
+            live = [i for i, r in enumerate(reqs) if len(r) > 3]
+            lg, _ = m.step_batch([states[i] for i in live], [[reqs[i][len(reqs[i]) - 3 + step]] for i in live], [[0]] * len(live))
+            for row, i in zip(lg, live):
+                got[i].append(row)
+        for i in range(len(reqs)):
+            assert np.abs(np.stack(got[i]) - alone[i]).max() < 2e-4 * np.abs(alone[i]).max(), (round_, i)
+            assert O.logit_error(np.stack(got[i])[-1:], O.forward(cfg, W, reqs[i])[0][-1:]).max() < TOL[True]
+        for st in states:
+            st.reset()
+    for st in pool:
+        st.close()
+
+
+def test_more_requests_than_a_pass_carries_and_prompts_longer_than_a_pass(hip_ctx, tmp_path):
+    cfg = O.config(vocab=31, width=16, loop=(0, 2, 2), side_dim=2, layers=[
+        O.rglru_layer(16, 2, 4, mlp=None),
+        O.latent_layer(2, 4, 4, 8, 8, O.rot(4, 1e4), mlp=O.dense(8)),
+        O.attention_layer(2, 1, 8, 8, O.rot(4, 1e4), mlp=None)])
+    W, m = make(hip_ctx, tmp_path, cfg, 21, ctx_len=3000)
+    reqs = [prompt(cfg, n, n) for n in (9, 2100, 4, 30, 2)]  # 2100 > one pass of 2048 rows; five requests > two per pass
+    states = [m.new_state() for _ in reqs]
+    lg, sampled = m.step_batch(states, reqs, [[len(r) - 1] for r in reqs], sample=True)
+    for i, r in enumerate(reqs):
+        want = O.forward(cfg, W, r)[0][-1:]
+        assert O.logit_error(lg[i:i + 1], want).max() < (TOL[True] if len(r) < 200 else 2e-4), i
+        assert len(r) > 200 or int(sampled[i]) == int(np.argmax(want))
+        assert states[i].context_length == len(r)
+    # the long prompt: against the same prompt through two explicit portions
+    st = m.new_state()
+    m.step_batch([st], [reqs[1][:1500]], [[]])
+    two, _ = m.step_batch([st], [reqs[1][1500:]], [[599]])
+    assert np.abs(two[0] - lg[1]).max() < 2e-4 * np.abs(two).max()
+    m.close()
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_long_decoding(models, full):
+    cfg, W, ms = models["b"]
+    m = ms[full]
+    toks = prompt(cfg, 230, 5)
+    want, _ = O.forward(cfg, W, toks)
+    st = m.new_state()
+    m.step_batch([st], [toks[:10]], [[]])
+    rows = [m.step_batch([st], [[t]], [[0]])[0][0] for t in toks[10:]]  # 220 decoded tokens across the key blocks' borders
+    assert rows_ok(O.logit_error(np.stack(rows), want[10:]), full)
+    st.close()
+
+
+def _match_queries_to_keys(W, cfg):
+    """Make a token's query point at the same token's key, so that one far key stands out of hundreds: latent attention gets query rows = (key up-projection) x
+    (down projection), grouped attention gets each group's key rows = the rows of its first query head."""
+    mx = cfg["layers"][0]["mixer"]
+    if cfg["layers"][0]["type"] == "latent_attention":
+        H, dim, rd, rank = mx["heads"], mx["dim"], mx["rot_dim"], mx["kv_rank"]
+        q = W["l0.mix.q"].reshape(H, dim + rd, -1).copy()
+        uk = W["l0.mix.uk"].reshape(H, dim, rank)
+        for a in range(H):
+            q[a, :dim] = uk[a] @ W["l0.mix.dkv"][:rank]
+        W["l0.mix.q"] = O.to_bf16(q.reshape(H * (dim + rd), -1))
+    else:
+        H, G, dim = mx["heads"], mx["kv_heads"], mx["dim"]
+        q, k = W["l0.mix.q"].reshape(H, dim, -1), W["l0.mix.k"].reshape(G, dim, -1).copy()
+        for g in range(G):
+            k[g] = q[g * (H // G)]
+        W["l0.mix.k"] = O.to_bf16(k.reshape(G * dim, -1))
+
+
+@pytest.mark.parametrize("kind", ["latent", "grouped"])
+def test_a_far_key_among_hundreds_decides_the_logits(hip_ctx, tmp_path, kind):
+    """The last token of a 700-token prompt also stands at position 2 and nowhere else, and queries are made to point at the keys of their own token: that one far
+    key takes a visible share of the softmax.  Replacing it must move the last logits exactly as the oracle says, in a whole prompt and when the tail is decoded
+    token by token -- a key that is dropped, doubled, rotated by a wrong position or read from a neighbouring row shows."""
+    layer = O.latent_layer(2, 8, 8, 8, 16, O.rot(8, 1e5), scale=0.03) if kind == "latent" else O.attention_layer(4, 2, 16, 8, O.rot(8, 1e5), scale=0.1)
+    cfg = O.config(vocab=41, width=32, layers=[layer])
+    W, m = make(hip_ctx, tmp_path, cfg, 8, ctx_len=1024, edit=lambda W: _match_queries_to_keys(W, cfg))
+    base = [int(t) for t in np.random.default_rng(4).integers(0, 39, size=700)]  # tokens 39 and 40 are kept for the marked positions
+    base[2] = base[-1] = 39
+    other = list(base)
+    other[2] = 40
+    want = [O.forward(cfg, W, t)[0][-1] for t in (base, other)]
+    assert O.logit_error(want[0][None], want[1][None]).max() > 50 * TOL[True], "the oracle itself does not see the token"
+    for toks, ref in zip((base, other), want):
+        st = m.new_state()
+        whole, _ = m.step_batch([st], [toks], [[699]])
+        st.reset()
+        m.step_batch([st], [toks[:640]], [[]])
+        for t in toks[640:-1]:
+            m.step_batch([st], [[t]], [[]])
+        dec, _ = m.step_batch([st], [[toks[-1]]], [[0]])
+        assert O.logit_error(whole, ref[None]).max() < TOL[True] and O.logit_error(dec, ref[None]).max() < TOL[True]
+        st.close()
+    m.close()
+
+
+def test_a_far_token_reaches_the_logits_only_through_the_recurrent_state(hip_ctx, tmp_path):
+    """No attention anywhere: what position 3 leaves at position 400 travels in the recurrent state alone (slow decays), through a prompt's pieces, through
+    portions and through decoded tokens."""
+    cfg = O.config(vocab=41, width=32, layers=[O.rglru_layer(32, 2, 3, mlp=None), O.rglru_layer(24, 3, 2, mlp=O.dense(16))])
+
+    def slow(W):
+        for i in (0, 1):
+            W[f"l{i}.mix.lam"] = O.to_bf16(np.full_like(W[f"l{i}.mix.lam"], -9.0) + 0.5 * (np.arange(W[f"l{i}.mix.lam"].size) % 3))
+    W, m = make(hip_ctx, tmp_path, cfg, 8, ctx_len=512, edit=slow)
+    base = prompt(cfg, 401, 4)
+    other = list(base)
+    other[3] = (base[3] + 7) % cfg["vocab"]
+    want = [O.forward(cfg, W, t)[0][-1] for t in (base, other)]
+    assert O.logit_error(want[0][None], want[1][None]).max() > 1e-3, "the oracle itself does not carry the token: slow the decays"
+    for toks, ref in zip((base, other), want):
+        st = m.new_state()
+        whole, _ = m.step_batch([st], [toks], [[400]])
+        st.reset()
+        m.step_batch([st], [toks[:100]], [[]])
+        m.step_batch([st], [toks[100:102]], [[]])
+        for t in toks[102:-1]:
+            m.step_batch([st], [[t]], [[]])
+        dec, _ = m.step_batch([st], [[toks[-1]]], [[0]])
+        assert O.logit_error(whole, ref[None]).max() < TOL[True] and O.logit_error(dec, ref[None]).max() < TOL[True]
+        st.close()
+    m.close()
+
+
+def test_the_first_tokens_and_a_state_that_held_another_request(models):
+    """Positions 0, 1, 2 of a sequence: zeros in front of the convolution, a zero recurrent state, one-key softmaxes -- also on a state that another, longer
+    request has just left (reset): nothing of it may be read."""
+    cfg, W, ms = models["a"]
+    m = ms[True]
+    st = m.new_state()
+    m.step_batch([st], [prompt(cfg, 80, 9)], [[]])
+    for n, seed in ((1, 1), (2, 2), (3, 3)):
+        st.reset()
+        toks = prompt(cfg, n, seed)
+        got, _ = m.step_batch([st], [toks], [list(range(n))])
+        assert O.logit_error(got, O.forward(cfg, W, toks)[0]).max() < TOL[True]
+    st.reset()
+    toks = prompt(cfg, 4, 7)
+    rows = [m.step_batch([st], [[t]], [[0]])[0][0] for t in toks]
+    assert O.logit_error(np.stack(rows), O.forward(cfg, W, toks)[0]).max() < TOL[True]
+    st.close()
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_greedy_generation_through_prefill_and_decode(models, name):
+    """The engine's own entry points: HipModel.prefill + chained decode (the sampled token is fed back on the device), then the stochastic sampler's plumbing."""
+    cfg, W, ms = models[name]
+    m = ms[True]
+    p = prompt(cfg, 25, 7)
+    m.reset()
+    m.set_sampling(None)
+    first = m.prefill(np.asarray(p, dtype=np.uint32))
+    rest, _ = m.decode(9)
+    got = [int(first)] + [int(t) for t in rest]
+    want, margin_ok = [], True
+    toks = list(p)
+    for _ in range(10):
+        row = O.forward(cfg, W, toks)[0][-1]
+        top2 = np.sort(row)[-2:]
+        margin_ok = margin_ok and (top2[1] - top2[0]) > 1e-3 * np.abs(row).max()
+        want.append(int(np.argmax(row)))
+        toks.append(want[-1])
+    assert margin_ok, "the oracle's own greedy stream has a near tie: pick another seed"
+    assert got == want and m.context_length == len(p) + 9
+    assert np.argmax(m.read_logits_f32()) == want[-1]
+    m.reset()
+    m.set_sampling(seed=3, temperature=1e-4)  # temperature -> 0 of the stochastic sampler is greedy
+    s1 = [int(m.prefill(np.asarray(p, dtype=np.uint32)))] + [int(t) for t in m.decode(4)[0]]
+    assert s1 == want[:5]
+    m.set_sampling(None)
+    m.reset()
+
+
+def test_generate_loop_of_the_text_front_end_and_the_pool(hip_ctx, tmp_path):
+    """LanguageModel.generate on a directory without tokenizer.json, and SequencePool.generate: prompts of unequal length prefilled in one batch and decoded
+    together, requests leaving as they finish (one by a stop token), their states reused by a second round -- against each prompt generated alone by the oracle"""
+    from uzu_amd.language_model import LanguageModel
+    from uzu_amd.serving import SequencePool
+    cfg = cfg_a()
+    W = O.weights(cfg, 31, logit_gain=3.0)
+    O.write_model_dir(str(tmp_path / "g"), cfg, W)
+    W64 = {k: v.astype(np.float64) for k, v in W.items()}
+    lm = LanguageModel(hip_ctx, str(tmp_path / "g"), max_context_length=128, flags=MODEL_FULL_F32, tokenizer_required=False)
+    p = prompt(cfg, 12, 3)
+    res = lm.generate(p, max_tokens=11, chunk=4)
+    assert res.token_ids == O.greedy(cfg, W64, p, 11) and res.prompt_tokens == 12
+    lm.close()
+    m = HipModel(hip_ctx, loader.load_model_dir(str(tmp_path / "g"), max_context_length=128), MODEL_BATCH(4) | MODEL_FULL_F32)
+    prompts = {"x": prompt(cfg, 3, 41), "y": prompt(cfg, 40, 42), "z": prompt(cfg, 17, 43)}
+    want = {k: O.greedy(cfg, W64, q, 8) for k, q in prompts.items()}
+    stop = want["y"][4]
+    cut = lambda seq: seq[:seq.index(stop)] if stop in seq else seq
+    pool = SequencePool(m)
+    for _ in range(2):
+        got = pool.generate(prompts, max_tokens=8, stop_token_ids=[stop])
+        assert got == {k: cut(v) for k, v in want.items()}
+        assert not pool.live and len(pool.free) == 3
+    pool.close()
+    m.close()
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_decode_graph_replays_equal_plain_launches(hip_ctx, tmp_path, full):
+    """The chained decode step is ONE captured hipGraph per state that reads its position from device memory.  Replayed in several calls, with eager batched
+    steps of OTHER states (which overwrite the model's pass tables) and synchronisations between them, every token and the logits after every call must equal
+    those of a model that decodes with plain launches."""
+    from uzu_amd.engine import MODEL_NO_GRAPH
+    cfg = cfg_b()
+    W = O.weights(cfg, 77)
+    O.write_model_dir(str(tmp_path / "m"), cfg, W)
+    bundle = loader.load_model_dir(str(tmp_path / "m"), max_context_length=256)
+    base = MODEL_BATCH(4) | (MODEL_FULL_F32 if full else 0)
+    graph, plain = HipModel(hip_ctx, bundle, base), HipModel(hip_ctx, bundle, base | MODEL_NO_GRAPH)
+    p, other = prompt(cfg, 70, 8), prompt(cfg, 33, 9)
+    firsts = [m.prefill(np.asarray(p, dtype=np.uint32)) for m in (graph, plain)]
+    assert firsts[0] == firsts[1]
+    side = [m.new_state() for m in (graph, plain)]
+    for call in range(4):
+        toks = [m.decode(5)[0] for m in (graph, plain)]
+        assert list(toks[0]) == list(toks[1]), call
+        assert np.array_equal(graph.read_logits_f32(), plain.read_logits_f32()), call
+        for m, st in zip((graph, plain), side):  # eager work on another state between the replays
+            m.step_batch([st], [other[call * 8:(call + 1) * 8]], [[7]])
+    assert graph.context_length == 70 + 20
+    for m in (graph, plain):
+        m.close()
+
+
+def test_refusals_of_the_engine(hip_ctx, tmp_path):
+    """what the engine does not run it refuses at creation, by name"""
+    import dataclasses
+    from uzu_amd import _ffi
+    cfg = cfg_b()
+    O.write_model_dir(str(tmp_path / "m"), cfg, O.weights(cfg, 3))
+    bundle = loader.load_model_dir(str(tmp_path / "m"), max_context_length=64)
+    broken = dataclasses.replace(bundle, layers=[dataclasses.replace(bundle.layers[0], layer_scale_mixer=bundle.layers[0].layer_scale_mixer, post_mixer_norm=type(bundle.layers[0].post_mixer_norm)(present=False))] + bundle.layers[1:])
+    with pytest.raises(_ffi.UzuHipError, match="layer scale follows a post norm"):
+        HipModel(hip_ctx, broken, MODEL_FULL_F32)
+    bf16 = dataclasses.replace(bundle, f32_stream=False)
+    with pytest.raises(_ffi.UzuHipError):
+        HipModel(hip_ctx, bf16, 0)

@@ -12,7 +12,7 @@ Prints ONE JSON line on rank 0 (contract in the task statement) with two extra o
   roofline     -- the dominant kernel (the int4 GEMV family) : algorithmic bytes / HIP-event time, vs 8 TB/s HBM
   cpu_baseline -- the CPU oracle (port of the reference's single-threaded CPU backend) timed on this host
 
-Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix | relulix (prefill / chained decode / batched
+Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix | relulix | begasun (prefill / chained decode / batched
 decode of an f32-stream design at real layer sizes beside the engine's closest existing model at equal sizes).
 """
 import argparse
@@ -59,10 +59,11 @@ def parse_args():
                     help="BASELINE.json configs[1..4]: c2 (default, the headline) Qwen3.5-0.8B int4 ctx-2048 decode; c3 Llama-3-8B int4, 4k prefill x 8 "
                          "sequences in batched passes (prefill tokens/s, MFMA roofline); c4 Llama-3-8B int8 decode (TP = --gpus); c5 Qwen3-14B-class int4 at "
                          "ctx 8192, one sequence decoding while another is prefilled (TP = --gpus)")
-    ap.add_argument("--design", choices=["", "lazolix", "relulix"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
+    ap.add_argument("--design", choices=["", "lazolix", "relulix", "begasun"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
                     "chained decode and batched decode of the f32-stream design at layer sizes of real models (random weights), beside the closest "
                     "bf16-stream model of the engine at equal sizes (windowed attention with sinks + int4 dense / bf16 expert MLPs); `relulix` does the same for the "
-                    "design of parallel blocks with rotated attention, retention layers and clamped experts, beside Lazolix with experts at equal sizes")
+                    "design of parallel blocks with rotated attention, retention layers and clamped experts, beside Lazolix with experts at equal sizes; `begasun` for the looped stack of recurrent units, latent attention with a rotated key part "
+                    "and grouped attention, beside Lazolix with dense blocks at equal sizes")
     ap.add_argument("--design-sizes", default="w1024,w2048", help="--design: comma-separated size presets")
     ap.add_argument("--sequences", type=int, default=8, help="c3: sequences per batched prefill pass")
     ap.add_argument("--prompt", type=int, default=4096, help="c3: prompt tokens per sequence")
@@ -601,8 +602,45 @@ def bench_relulix(args):
     print(json.dumps(out), flush=True)
 
 
+def bench_begasun(args):
+    """Prefill / decode throughput of Begasun models (a recurrent layer and a latent-attention layer run twice as a loop, then a grouped-attention layer and a second
+    latent-attention layer; norms on both sides of every sublayer, layer scales, the per-layer token input, clamped dense blocks) beside the closest existing model
+    at equal size: Lazolix with dense blocks (the f32-stream design with latent attention: same width / heads / head widths / cache row width / dense width /
+    vocabulary, as many layers as Begasun has layer runs).  One JSON line."""
+    import tempfile
+    from uzu_amd import begasun, loader, synthetic as S
+    from uzu_amd.backend import Context
+    ctx = Context.new(0)
+    prompt_len, steps, warm, nbatch = 2048, max(8, min(args.steps, 128)), max(2, min(args.warmup, 8)), 8
+    out = {"metric": "begasun_side_run", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 products, f32 stream", "data": "synthetic (random weights, synthetic token ids)",
+           "prompt_tokens": prompt_len, "decode_steps": steps, "batched_decode_sequences": nbatch, "sizes": {}}
+    for size in [s for s in args.design_sizes.split(",") if s]:
+        z = LAZOLIX_SIZES[size]
+        prompt = S.synthetic_prompt(prompt_len, z["vocab"]).astype(np.uint32)
+        context = prompt_len + steps + warm + 64
+        H, G, dim, vd, rot_dim = z["heads"], max(1, z["heads"] // 4), z["dim"], z["vdim"], 64
+        rank = z["rank"] - rot_dim  # the cache row [latent | rotated part] is as wide as the closest model's latent
+        yarn = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+        mlp = begasun.dense_mlp(z["ff"], limit=7.0)
+        lat = lambda: begasun.latent_attention_layer(H, dim, rot_dim, vd, rank, begasun.rotation(rot_dim, 10000.0, yarn), mlp=mlp)
+        layers = [begasun.rglru_layer(z["width"], H, 4, mlp=mlp), lat(), begasun.attention_layer(H, G, dim, vd, begasun.rotation(dim // 2, 10000.0), mlp=mlp), lat()]
+        cfg = begasun.config(z["vocab"], z["width"], layers, loop=(0, 2, 2), side_dim=256)
+        with tempfile.TemporaryDirectory() as tmp:
+            begasun.save(tmp, cfg, begasun.random_tensors(cfg, seed=1))
+            bundle = loader.load_model_dir(tmp, max_context_length=context)
+        runs = len(bundle.layers)
+        rec = {"begasun": _time_f32_stream(ctx, bundle, prompt, steps, warm, nbatch),
+               "closest_dense": _time_f32_stream(ctx, _lazolix_bundle(dict(z, layers=runs), "dense", context), prompt, steps, warm, nbatch)}
+        out["sizes"][size] = {"shape": dict(z, kv_heads=G, kv_rank=rank, rot_dim=rot_dim, lru_width=z["width"], lru_blocks=H, conv=4, side_dim=256, layer_runs=runs,
+                                            pattern="loop x 2 (recurrent unit, latent attention), grouped attention, latent attention"), **rec}
+    ctx.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
+    if args.design == "begasun":
+        return bench_begasun(args)
     if args.design == "lazolix":
         return bench_lazolix(args)
     if args.design == "relulix":

@@ -67,6 +67,8 @@ struct Stream32 {
     float alpha_out = 0.f;
     float* ret_ws = nullptr; // retention in chunks: one state block per (chunk of the pass, head)
     size_t ret_ws_bytes = 0;
+    float* lru_ws = nullptr; // the recurrent unit in pieces: local state, decay product and carry per (piece of the pass, channel)
+    size_t lru_ws_bytes = 0;
     float* att_ws = nullptr; // partial sums of the key-split attention of decode-sized passes
     size_t att_ws_bytes = 0;
     float* taps = nullptr; // UZU_MODEL_DEBUG_TAPS: f32 [layers][max_rows][d], what each layer handed on in the last pass
@@ -234,6 +236,8 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             gp.branches = S.q, gp.ld = L.qkv.n, gp.x_col = w, gp.u = S.lru_u, gp.gates = S.lru_g, gp.out = S.attn, gp.conv_w = L.conv_w, gp.conv_b = L.conv_b, gp.gate_b = X.lru_gate_b;
             gp.lambda = X.lru_lambda, gp.rate = h.lru_decay_rate, gp.states = (float* const*)caches, gp.conv_states = (float* const*)(S.d_cache2_ptrs + (size_t)l * S.max_seqs);
             gp.spans = S.d_spans, gp.row_seq = S.d_row_seq, gp.nseq = nseq, gp.rows = rows, gp.width = w, gp.blocks = h.lru_blocks, gp.taps = h.dn_kernel_size, gp.max_count = max_count;
+            for (uint32_t i = 0; i < nseq; ++i) gp.pieces += (counts[i] + 31) / 32;
+            gp.piece_ws = S.lru_ws, gp.piece_ws_bytes = S.lru_ws_bytes;
             RUN("lru_conv", (size_t)rows * w * 4 * (gp.taps + 1), k::lru_conv(s, gp));
             {   // both gates of every block in one batched product; what enters the recurrence is never rounded: true f32 products in both precisions
                 k::LinearF32Params p{};
@@ -808,6 +812,10 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             S.ret_ws_bytes = std::max(S.ret_ws_bytes, k::retention_chunk_ws_bytes(S.max_rows / 64 + S.max_seqs, h.num_heads, h.head_dim, h.value_head_dim));
     }
     if (S.ret_ws_bytes) TRY(need_f32(m, S.ret_ws_bytes / 4, &S.ret_ws));
+    if (w_lru) {
+        S.lru_ws_bytes = k::lru_piece_ws_bytes(S.max_rows / 32 + S.max_seqs, w_lru);
+        TRY(need_f32(m, S.lru_ws_bytes / 4, &S.lru_ws));
+    }
     TRY(dev_alloc(m, k::argmax_scratch_bytes(1), &m->argmax_scratch));
     TRY(dev_alloc(m, k::unified_sampling_scratch_bytes(1), &m->sampling_scratch));
     TRY(dev_alloc(m, 8, &p, true)); m->d_seed = (uint64_t*)p;

@@ -3,8 +3,9 @@
 //
 // The recurrence is element-wise per channel and linear in S, so a sequence's rows can be cut into pieces: a piece scanned from zero yields its local states L_t
 // and decay products P_t = a_(first) ... a_t, and the true state is S_t = L_t + P_t * (the state in front of the piece).  The position-by-position form walks a
-// sequence's rows in one thread per channel (decode steps, short portions); the pieced form spreads a long prompt's rows over 16 threads per channel and joins
-// the pieces' carries in order.  Both leave S and the convolution's last taps - 1 inputs in the sequence's state.
+// sequence's rows in one thread per channel (decode steps, short portions); the pieced form cuts a prompt's rows into pieces of 32, scans every piece from zero
+// in its own thread, joins the pieces' carries in order and walks the pieces again from their true carries (three launches that fill the chip).  Both leave S and
+// the convolution's last taps - 1 inputs in the sequence's state.
 #include "device_utils.h"
 #include "kernels_stream32.h"
 
@@ -81,50 +82,72 @@ __global__ void __launch_bounds__(256) lru_scan_steps_kernel(GatedLruParams p) {
     conv_state_update(p, sp, z, c);
 }
 
-// in pieces: workgroup = (sequence, 16 channels), thread = (piece of the sequence's rows, channel); 16 pieces.  Pass 1 scans a piece from zero (L, P at its end),
-// the carries are joined in piece order through LDS, pass 2 walks the piece again from its true carry and writes the rows.
-constexpr uint32_t kPieces = 16, kChan = 16;
-__global__ void __launch_bounds__(256) lru_scan_pieces_kernel(GatedLruParams p) {
-    __shared__ float s_L[kPieces][kChan], s_P[kPieces][kChan], s_in[kPieces][kChan];
-    const uint32_t z = blockIdx.x, cl = threadIdx.x & (kChan - 1), piece = threadIdx.x / kChan;
-    const uint32_t c = blockIdx.y * kChan + cl;
-    const bool on = c < p.width;
-    const SeqSpan sp = p.spans[z];
-    const uint32_t per = (sp.count + kPieces - 1) / kPieces;
-    const uint32_t i0 = piece * per < sp.count ? piece * per : sp.count, i1 = i0 + per < sp.count ? i0 + per : sp.count;
-    const uint32_t bw = p.width / p.blocks, blk = on ? c / bw : 0, o = on ? c - blk * bw : 0;
-    float sl = 0.0f, br = 0.0f, bi = 0.0f;
-    if (on) {
-        sl = p.rate * softplus_f32(p.lambda[c]);
-        if (p.gate_b) br = p.gate_b[(size_t)blk * 2 * bw + o], bi = p.gate_b[(size_t)blk * 2 * bw + bw + o];
+// In pieces of kPieceRows rows: thread = (piece, channel), consecutive lanes on consecutive channels, so that a prompt's rows fill the chip.
+//   local:  a piece scanned from zero: L (its last local state) and P (the product of its decays) per channel
+//   carry:  thread = (sequence, channel) joins the pieces in order: the state in front of every piece, the sequence's state behind the pass, the convolution's window
+//   out:    the piece again from its true carry; writes the rows
+constexpr uint32_t kPieceRows = 32;
+// piece g of the pass -> its sequence, first row (within the sequence's share) and row count; false behind the last piece
+__device__ __forceinline__ bool piece_of(const GatedLruParams& p, uint32_t g, SeqSpan& sp, uint32_t& i0, uint32_t& n) {
+    for (uint32_t z = 0; z < p.nseq; ++z) {
+        sp = p.spans[z];
+        const uint32_t np = (sp.count + kPieceRows - 1) / kPieceRows;
+        if (g < np) {
+            i0 = g * kPieceRows;
+            n = sp.count - i0 < kPieceRows ? sp.count - i0 : kPieceRows;
+            return true;
+        }
+        g -= np;
     }
-    float L = 0.0f, P = 1.0f;
-    if (on)
-        for (uint32_t i = i0; i < i1; ++i) {
-            const Coef k = coef_of(p, sp.row0 + i, c, bw, blk, o, sl, br, bi);
+    return false;
+}
+
+template <bool OUT>
+__global__ void __launch_bounds__(256) lru_piece_kernel(GatedLruParams p) {
+    const uint32_t g = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= p.width) return;
+    SeqSpan sp;
+    uint32_t i0, n;
+    if (!piece_of(p, g, sp, i0, n)) return;
+    const uint32_t bw = p.width / p.blocks, blk = c / bw, o = c - blk * bw;
+    const float sl = p.rate * softplus_f32(p.lambda[c]);
+    const float br = p.gate_b ? p.gate_b[(size_t)blk * 2 * bw + o] : 0.0f, bi = p.gate_b ? p.gate_b[(size_t)blk * 2 * bw + bw + o] : 0.0f;
+    const size_t at = (size_t)g * p.width + c;
+    if (!OUT) {
+        float L = 0.0f, P = 1.0f;
+        for (uint32_t i = 0; i < n; ++i) {
+            const Coef k = coef_of(p, sp.row0 + i0 + i, c, bw, blk, o, sl, br, bi);
             L = fmaf(k.a, L, k.b);
             P *= k.a;
         }
-    s_L[piece][cl] = L, s_P[piece][cl] = P;
-    __syncthreads();
-    if (piece == 0 && on) {
-        float S = sp.start ? p.states[z][c] : 0.0f;
-        for (uint32_t q = 0; q < kPieces; ++q) {
-            s_in[q][cl] = S;
-            S = fmaf(s_P[q][cl], S, s_L[q][cl]);
+        p.piece_ws[at] = L, p.piece_ws[(size_t)p.pieces * p.width + at] = P;
+    } else {
+        float S = p.piece_ws[(size_t)2 * p.pieces * p.width + at];
+        for (uint32_t i = 0; i < n; ++i) {
+            const uint32_t r = sp.row0 + i0 + i;
+            const Coef k = coef_of(p, r, c, bw, blk, o, sl, br, bi);
+            S = fmaf(k.a, S, k.b);
+            p.out[(size_t)r * p.width + c] = S * gelu_tanh(p.branches[(size_t)r * p.ld + c]);
         }
-        p.states[z][c] = S;
     }
-    __syncthreads();
-    if (!on) return;
-    float S = s_in[piece][cl];
-    for (uint32_t i = i0; i < i1; ++i) {
-        const uint32_t r = sp.row0 + i;
-        const Coef k = coef_of(p, r, c, bw, blk, o, sl, br, bi);
-        S = fmaf(k.a, S, k.b);
-        p.out[(size_t)r * p.width + c] = S * gelu_tanh(p.branches[(size_t)r * p.ld + c]);
+}
+
+__global__ void __launch_bounds__(256) lru_piece_carry_kernel(GatedLruParams p) {
+    const uint32_t z = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= p.width) return;
+    uint32_t g = 0;
+    for (uint32_t q = 0; q < z; ++q) g += (p.spans[q].count + kPieceRows - 1) / kPieceRows;
+    const SeqSpan sp = p.spans[z];
+    const uint32_t np = (sp.count + kPieceRows - 1) / kPieceRows;
+    const size_t plane = (size_t)p.pieces * p.width;
+    float S = sp.start ? p.states[z][c] : 0.0f;
+    for (uint32_t q = 0; q < np; ++q) {
+        const size_t at = (size_t)(g + q) * p.width + c;
+        p.piece_ws[2 * plane + at] = S;
+        S = fmaf(p.piece_ws[plane + at], S, p.piece_ws[at]);
     }
-    if (piece == 0) conv_state_update(p, sp, z, c);
+    p.states[z][c] = S;
+    conv_state_update(p, sp, z, c);
 }
 
 uzu_status lru_check(const GatedLruParams& p) {
@@ -136,6 +159,8 @@ uzu_status lru_check(const GatedLruParams& p) {
 
 } // namespace
 
+size_t lru_piece_ws_bytes(uint32_t pieces, uint32_t width) { return (size_t)3 * pieces * width * 4; }
+
 uzu_status lru_conv(hipStream_t s, const GatedLruParams& p) {
     if (!p.rows) return UZU_OK;
     UZU_PROPAGATE(lru_check(p));
@@ -146,8 +171,14 @@ uzu_status lru_scan(hipStream_t s, const GatedLruParams& p) {
     if (!p.rows) return UZU_OK;
     UZU_PROPAGATE(lru_check(p));
     UZU_REQUIRE(p.gates && p.out && p.lambda && p.states && p.nseq, "gated_lru: null argument");
-    const bool pieces = p.form == 2 || (p.form == 0 && p.max_count >= 64);
-    if (pieces) return launch_check([&] { hipLaunchKernelGGL(lru_scan_pieces_kernel, dim3(p.nseq, (p.width + kChan - 1) / kChan), dim3(256), 0, s, p); }, "lru_scan_pieces");
+    const bool have_ws = p.piece_ws && p.pieces && lru_piece_ws_bytes(p.pieces, p.width) <= p.piece_ws_bytes;
+    UZU_REQUIRE(p.form != 2 || have_ws, "gated_lru: the pieced form needs its piece count and workspace");
+    if (p.form == 2 || (p.form == 0 && have_ws && p.max_count >= 2 * kPieceRows)) {
+        const dim3 grid(p.pieces, (p.width + 255) / 256);
+        UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(lru_piece_kernel<false>, grid, dim3(256), 0, s, p); }, "lru_piece_local"));
+        UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(lru_piece_carry_kernel, dim3(p.nseq, (p.width + 255) / 256), dim3(256), 0, s, p); }, "lru_piece_carry"));
+        return launch_check([&] { hipLaunchKernelGGL(lru_piece_kernel<true>, grid, dim3(256), 0, s, p); }, "lru_piece_out");
+    }
     return launch_check([&] { hipLaunchKernelGGL(lru_scan_steps_kernel, dim3(p.nseq, (p.width + 255) / 256), dim3(256), 0, s, p); }, "lru_scan_steps");
 }
 

@@ -278,8 +278,9 @@ uzu_status head_rms_gate(hipStream_t s, float* x, const float* gate, uint32_t ld
 //   lru_scan:  with g = the gate pre-activations [rows][blocks][2 bw] (recurrence gate's bw numbers, then the input gate's) and their biases,
 //              a = exp(-rate * sigmoid(g_r + b_r) * softplus(lambda)),  S <- a S + sqrt(1 - a^2) * sigmoid(g_i + b_i) * u,  out[r, c] = S * gelu_tanh(gate branch);
 //              S starts from the sequence's state (zero at position 0) and is left there behind the pass's last row, and so are the last taps - 1 inputs.
-//              All f32.  form 0: chosen by the row count; 1: position by position; 2: in pieces of a sequence's rows, each scanned from zero with its decay product,
-//              the pieces' carries joined in order (differs from form 1 by f32 rounding only).
+//              All f32.  form 0: chosen by the row count; 1: position by position; 2: in pieces of 32 rows, each scanned from zero with its decay product,
+//              the pieces' carries joined in order (differs from form 1 by f32 rounding only); needs `pieces` = sum over the sequences of ceil(count / 32) and a
+//              workspace of lru_piece_ws_bytes(pieces, width) bytes, without which form 0 goes position by position.
 struct GatedLruParams {
     const float* branches;
     uint32_t ld, x_col;
@@ -295,7 +296,11 @@ struct GatedLruParams {
     uint32_t nseq, rows, width, blocks, taps;
     uint32_t form;
     uint32_t max_count; // the longest sequence share of the pass (the caller knows the counts)
+    uint32_t pieces;
+    float* piece_ws;
+    size_t piece_ws_bytes;
 };
+size_t lru_piece_ws_bytes(uint32_t pieces, uint32_t width);
 uzu_status lru_conv(hipStream_t s, const GatedLruParams& p);
 uzu_status lru_scan(hipStream_t s, const GatedLruParams& p);
 

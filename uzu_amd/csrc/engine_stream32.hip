@@ -207,6 +207,14 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     const float* cur = S.slots; // what the layer about to run reads: X_0, then the depth mix of the layer before
     uint32_t max_count = 0;
     for (uint32_t c : counts) max_count = std::max(max_count, c);
+    // A sublayer's result joins the stream behind its post norm; the same launch leaves the norm of the new rows for the sublayer that follows where that is an
+    // RMS norm with a weight vector (`next`), so that norm needs no launch of its own.
+    auto add_normed = [&](const float* y, const float* residual, float* out, const DNorm& N, const float* layer_scale, const DNorm* next) {
+        RUN("rms_norm_add_rows", (size_t)rows * d * (next ? 16 : 12),
+            k::rms_norm_add_rows(s, y, residual, out, N.scales, N.offset, layer_scale, N.eps, rows, d, next ? S.normed : nullptr, next ? next->scales : nullptr,
+                                 next ? next->offset : 0.0f, next ? next->eps : 0.0f));
+    };
+    bool normed_ready = false; // S.normed already holds this run's pre-mixer norm (left by the run before)
     for (uint32_t l = 0; l < nl; ++l) {
         DLayer& L = m->layers[l];
         const Stream32::Layer& X = S.layers[l];
@@ -220,7 +228,14 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             run_linear(e, b);
             cur = S.xin;
         }
-        if (h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH) {
+        // which launch ends this run, and whether it can leave the next run's pre-mixer norm
+        const DNorm* next_pre = nullptr;
+        if (l + 1 < nl && !X.depth_weights && !S.layers[l + 1].reentry_a.w && m->layers[l + 1].d.pre_mixer_norm.kind == UZU_NORM_STATISTICS) next_pre = &m->layers[l + 1].pre_mixer;
+        const bool pre_mlp_fused = !h.no_mlp && !h.parallel_block && L.post_mixer.present && h.pre_mlp_norm.kind == UZU_NORM_STATISTICS;
+        const bool have_normed = normed_ready;
+        normed_ready = false;
+        if (have_normed) {
+        } else if (h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH) {
             run_norm(e, L.pre_mixer, h.pre_mixer_norm.kind, X.alpha1, cur, S.normed, rows, d, nullptr);
         } else { // dynamic-tanh norm + token shift
             k::DynTanhParams np{};
@@ -333,7 +348,8 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         } // latent attention
         if (L.post_mixer.present) { // the mixer's result joins the stream behind its own norm (and the layer scale)
             run_linear(e, lin(S, L.out, S.attn, S.tmp, rows));
-            RUN("rms_norm_add_rows", (size_t)rows * d * 12, k::rms_norm_add_rows(s, S.tmp, cur, slot, L.post_mixer.scales, L.post_mixer.offset, X.ls1, L.post_mixer.eps, rows, d));
+            add_normed(S.tmp, cur, slot, L.post_mixer, X.ls1, pre_mlp_fused ? &L.pre_mlp : (h.no_mlp && !h.has_ple) ? next_pre : nullptr);
+            normed_ready = h.no_mlp && !h.has_ple && next_pre;
         } else { // X_(l+1) = input + out projection
             k::LinearF32Params p = lin(S, L.out, S.attn, slot, rows);
             p.residual = cur, p.ldr = d;
@@ -341,7 +357,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         }
         if (!h.no_mlp) {
             // a parallel block's MLP reads the rows the mixer read (still in S.normed) and adds to the same sum; otherwise the MLP has its own norm of the sum so far
-            if (!h.parallel_block) run_norm(e, L.pre_mlp, h.pre_mlp_norm.kind, X.alpha2, slot, S.normed, rows, d, nullptr);
+            if (!h.parallel_block && !pre_mlp_fused) run_norm(e, L.pre_mlp, h.pre_mlp_norm.kind, X.alpha2, slot, S.normed, rows, d, nullptr);
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
                 const uint32_t E = M.num_routed_experts, top = M.num_active_experts, ff = M.expert_hidden_dim;
@@ -374,7 +390,8 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
                 }
                 if (L.post_mlp.present) {
                     run_linear(e, lin(S, L.down, S.hid, S.tmp, rows));
-                    RUN("rms_norm_add_rows", (size_t)rows * d * 12, k::rms_norm_add_rows(s, S.tmp, slot, slot, L.post_mlp.scales, L.post_mlp.offset, X.ls2, L.post_mlp.eps, rows, d));
+                    add_normed(S.tmp, slot, slot, L.post_mlp, X.ls2, h.has_ple ? nullptr : next_pre);
+                    normed_ready = !h.has_ple && next_pre;
                 } else {
                     k::LinearF32Params down = lin(S, L.down, S.hid, slot, rows);
                     down.residual = slot, down.ldr = d;
@@ -383,11 +400,13 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             }
         }
         if (h.has_ple) { // the per-layer token input: x <- x + norm(projection(gelu(gate x) * the token's slice of the side table))
-            run_linear(e, lin(S, L.ple_gate, slot, S.side_g, rows));
-            RUN("side_gate_mul", (size_t)rows * h.ple_dim * 10, k::side_gate_mul(s, S.side_g, d_tokens, (const uint16_t*)m->ple_token_embedding.w, m->ple_token_embedding.k,
-                                                                              h.ple_slice * h.ple_dim, m->ple_token_embedding.n, rows, h.ple_dim));
+            k::LinearF32Params g = lin(S, L.ple_gate, slot, S.side_g, rows); // gelu and the token's slice in the product's epilogue
+            g.act = 2, g.mul_table = (const uint16_t*)m->ple_token_embedding.w, g.mul_tokens = d_tokens, g.mul_ld = m->ple_token_embedding.k, g.mul_col0 = h.ple_slice * h.ple_dim;
+            g.mul_vocab = m->ple_token_embedding.n;
+            run_linear(e, g);
             run_linear(e, lin(S, L.ple_projection, S.side_g, S.tmp, rows));
-            RUN("rms_norm_add_rows", (size_t)rows * d * 12, k::rms_norm_add_rows(s, S.tmp, slot, slot, L.ple_norm.scales, L.ple_norm.offset, nullptr, L.ple_norm.eps, rows, d));
+            add_normed(S.tmp, slot, slot, L.ple_norm, nullptr, next_pre);
+            normed_ready = next_pre != nullptr;
         }
         if (X.depth_weights) {
             RUN("depth_mix", (size_t)rows * d * 4 * (l + 3), k::depth_mix(s, S.slots, slot_stride, X.depth_weights, h.num_depth_weights, S.xin, rows, d));

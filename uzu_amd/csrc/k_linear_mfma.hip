@@ -129,6 +129,11 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
                 }
                 if (p.y_scale != 0.0f) v *= p.y_scale;
                 if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)row * p.ldgate + z]));
+                if (p.mul_table) {
+                    uint32_t t = p.mul_tokens[row];
+                    if (t >= p.mul_vocab) t = 0;
+                    v *= bf16_to_f32(p.mul_table[(size_t)t * p.mul_ld + p.mul_col0 + n]);
+                }
                 if (p.residual) v += p.residual[(size_t)row * p.ldr + n];
                 y[(size_t)row * p.ldy + n] = v;
             }

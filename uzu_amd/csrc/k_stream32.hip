@@ -69,8 +69,9 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, floa
 }
 
 // the same sum of squares over a sublayer's result y; the normed row joins the stream: out = residual + y * inv * (scales + offset) * layer_scale
+// ... and, with `next`, the norm of the new row for the sublayer that follows (its own weights, offset and epsilon): next[r] = rms(out[r]) * (next_scales + next_offset)
 __global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale,
-                                                                float eps, uint32_t d) {
+                                                                float eps, uint32_t d, float* next, const float* next_scales, float next_offset, float next_eps) {
     __shared__ float s_red[256];
     const uint32_t r = blockIdx.x;
     const float* yr = y + (size_t)r * d;
@@ -85,23 +86,28 @@ __global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, 
     const float inv = 1.0f / sqrtf(s_red[0] / (float)d + eps);
     const float* res = residual + (size_t)r * d;
     float* o = out + (size_t)r * d;
+    float acc2 = 0.0f;
     for (uint32_t i = threadIdx.x; i < d; i += 256) {
         float v = yr[i] * inv * (scales[i] + offset);
         if (layer_scale) v *= layer_scale[i];
-        o[i] = res[i] + v;
+        v = res[i] + v;
+        o[i] = v;
+        acc2 = fmaf(v, v, acc2);
     }
+    if (!next) return;
+    __syncthreads(); // s_red[0] has been read by everyone
+    s_red[threadIdx.x] = acc2;
+    __syncthreads();
+    for (uint32_t w = 128; w > 0; w >>= 1) {
+        if (threadIdx.x < w) s_red[threadIdx.x] += s_red[threadIdx.x + w];
+        __syncthreads();
+    }
+    const float inv2 = 1.0f / sqrtf(s_red[0] / (float)d + next_eps);
+    float* nx = next + (size_t)r * d;
+    for (uint32_t i = threadIdx.x; i < d; i += 256) nx[i] = o[i] * inv2 * (next_scales[i] + next_offset); // (the thread's own stores)
 }
 
 __device__ __forceinline__ float gelu_tanh_f32(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
-
-__global__ void __launch_bounds__(256) side_gate_mul_kernel(float* g, const uint32_t* tokens, const uint16_t* table, uint32_t table_ld, uint32_t col0, uint32_t vocab, uint32_t dim) {
-    const uint32_t r = blockIdx.x;
-    uint32_t t = tokens[r];
-    if (t >= vocab) t = 0;
-    const uint16_t* e = table + (size_t)t * table_ld + col0;
-    float* row = g + (size_t)r * dim;
-    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) row[i] = gelu_tanh_f32(row[i]) * bf16_to_f32(e[i]);
-}
 
 __global__ void __launch_bounds__(256) dyn_tanh_kernel(DynTanhParams p) {
     const uint32_t r = blockIdx.x;
@@ -160,6 +166,13 @@ __device__ __forceinline__ float apply_tail(float v, const LinearF32Params& p, u
     if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)r * p.ldgate + z]));
     return v;
 }
+// ... and a per-(row's token, column) multiplier from a bf16 table
+__device__ __forceinline__ float apply_token_mul(float v, const LinearF32Params& p, uint32_t r, uint32_t n) {
+    if (!p.mul_table) return v;
+    uint32_t t = p.mul_tokens[r];
+    if (t >= p.mul_vocab) t = 0;
+    return v * bf16_to_f32(p.mul_table[(size_t)t * p.mul_ld + p.mul_col0 + n]);
+}
 
 __global__ void __launch_bounds__(256) gated_act_rows_kernel(const float* y1, float* hidden, uint32_t ff, ExpertAct act) {
     const float* src = y1 + (size_t)blockIdx.x * 2 * ff;
@@ -214,7 +227,7 @@ __global__ void __launch_bounds__(256) linear_rows_kernel(LinearF32Params p, uin
         for (int i = 0; i < RT; ++i) {
             const uint32_t r = r0 + i;
             if (r >= p.rows) break;
-            float v = apply_tail(apply_act(acc[i] + bias, p.act), p, r, z);
+            float v = apply_token_mul(apply_tail(apply_act(acc[i] + bias, p.act), p, r, z), p, r, n);
             if (p.residual) v += p.residual[(size_t)r * p.ldr + n];
             y[(size_t)r * p.ldy + n] = v;
         }
@@ -269,7 +282,7 @@ __global__ void __launch_bounds__(256) linear_tile_kernel(LinearF32Params p) {
         for (int j = 0; j < 4; ++j) {
             const uint32_t n = n0 + tx * 4 + j;
             if (n >= p.n) continue;
-            float v = apply_tail(apply_act(acc[i][j] + (p.bias ? bf16_to_f32(p.bias[n]) : 0.0f), p.act), p, r, z);
+            float v = apply_token_mul(apply_tail(apply_act(acc[i][j] + (p.bias ? bf16_to_f32(p.bias[n]) : 0.0f), p.act), p, r, z), p, r, n);
             if (p.residual) v += p.residual[(size_t)r * p.ldr + n];
             y[(size_t)r * p.ldy + n] = v;
         }
@@ -502,23 +515,17 @@ uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float*
 }
 
 uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
-                             uint32_t rows, uint32_t d) {
+                             uint32_t rows, uint32_t d, float* next, const float* next_scales, float next_offset, float next_eps) {
     if (!rows) return UZU_OK;
-    UZU_REQUIRE(y && residual && out && scales && d, "rms_norm_add_rows: null argument");
-    return launch_check([&] { hipLaunchKernelGGL(rms_norm_add_rows_kernel, dim3(rows), dim3(256), 0, s, y, residual, out, scales, offset, layer_scale, eps, d); },
-                        "rms_norm_add_rows");
+    UZU_REQUIRE(y && residual && out && scales && d && (!next || next_scales), "rms_norm_add_rows: null argument");
+    return launch_check([&] { hipLaunchKernelGGL(rms_norm_add_rows_kernel, dim3(rows), dim3(256), 0, s, y, residual, out, scales, offset, layer_scale, eps, d, next, next_scales,
+                                                 next_offset, next_eps); }, "rms_norm_add_rows");
 }
 
 uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act) {
     if (!rows || !ff) return UZU_OK;
     UZU_REQUIRE(y1 && hidden, "gated_act_rows: null argument");
     return launch_check([&] { hipLaunchKernelGGL(gated_act_rows_kernel, dim3(rows), dim3(256), 0, s, y1, hidden, ff, act); }, "gated_act_rows");
-}
-
-uzu_status side_gate_mul(hipStream_t s, float* g, const uint32_t* tokens, const uint16_t* table, uint32_t table_ld, uint32_t col0, uint32_t vocab, uint32_t rows, uint32_t dim) {
-    if (!rows || !dim) return UZU_OK;
-    UZU_REQUIRE(g && tokens && table && col0 + dim <= table_ld, "side_gate_mul: null argument or a slice outside the table's rows");
-    return launch_check([&] { hipLaunchKernelGGL(side_gate_mul_kernel, dim3(rows), dim3(dim < 256 ? 64 : 256), 0, s, g, tokens, table, table_ld, col0, vocab, dim); }, "side_gate_mul");
 }
 
 uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p) {
@@ -542,6 +549,7 @@ uzu_status linear_f32(hipStream_t s, const LinearF32Params& p, const char** vari
     if (!p.rows || !p.n || !p.batch) return UZU_OK;
     UZU_REQUIRE(p.x && p.w && p.y && p.k, "linear_f32: null argument");
     UZU_REQUIRE(!p.residual || p.batch == 1, "linear_f32: a residual only with one product per launch");
+    UZU_REQUIRE(!p.mul_table || (p.mul_tokens && p.batch == 1 && !p.row_offsets && p.mul_col0 + p.n <= p.mul_ld), "linear_f32: a token multiplier needs the rows' tokens, one product, columns inside the table");
     UZU_REQUIRE(p.ldx >= p.k && p.ldy >= p.n && p.batch <= 65535, "linear_f32: row pitch below the row length");
     if (p.row_offsets || p.row_map) { // the grouped / gathered form lives in the matrix-core kernel only
         UZU_UNSUPPORTED(!linear_mfma_supported(p), "linear_f32: grouped / gathered rows need bf16 products and 8-aligned k");

@@ -32,9 +32,10 @@ uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float*
                          float offset = 0.0f);
 
 // A sublayer's result joins the stream behind its own norm:  out[r, :] = residual[r, :] + y[r, :] / sqrt(mean(y[r, :]^2) + eps) * (scales + offset) * layer_scale
-// (scales f32 [d]; layer_scale f32 [d] or null; out may alias residual).  The same fixed-order sum of squares as rms_norm_rows.
+// (scales f32 [d]; layer_scale f32 [d] or null; out may alias residual).  The same fixed-order sum of squares as rms_norm_rows.  With `next` the launch also leaves
+// the norm of the new row for the sublayer that follows: next[r, :] = out[r, :] / sqrt(mean(out[r, :]^2) + next_eps) * (next_scales + next_offset).
 uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
-                             uint32_t rows, uint32_t d);
+                             uint32_t rows, uint32_t d, float* next = nullptr, const float* next_scales = nullptr, float next_offset = 0.0f, float next_eps = 0.0f);
 
 // Dynamic-tanh norm, optionally followed by the token shift:
 //   h[r]   = tanh(alpha * x[src(r)]) * scales + biases          src(r) = row_index ? row_index[r] : r
@@ -77,6 +78,11 @@ struct LinearF32Params {
     float y_scale;     // != 0: the product (behind bias and act, before the residual) is multiplied by it
     const float* gate; // batched products: product z of row r is multiplied by sigmoid(gate[r * ldgate + z]) (a scalar gate per head); null = none
     uint32_t ldgate;
+    // a multiplier per (row's token, column) behind all of that: y[r, n] *= f32(mul_table[token[r] * mul_ld + mul_col0 + n])  (bf16 table, an id >= mul_vocab reads
+    // row 0; one product per launch; null = none) -- the gate of a per-layer token input
+    const uint16_t* mul_table;
+    const uint32_t* mul_tokens;
+    uint32_t mul_ld, mul_col0, mul_vocab;
     // Grouped form (matrix-core kernel only; the experts of a mixture, each with its own bucket of rows): product z covers rows row_offsets[z] ..
     // row_offsets[z + 1] - 1 of X and Y (device array [batch + 1]; x_batch / y_batch unused, `rows` = an upper bound of the total for the grid).
     const uint32_t* row_offsets;
@@ -104,8 +110,6 @@ struct ExpertAct {
 };
 // The gated product of a dense block: hidden[r, f] = act(gate = y1[r, ff + f], up = y1[r, f])   (y1 f32 [rows][2 ff]: up rows first, as the packed projection yields them)
 uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act);
-// Per-layer token input: g[r, j] <- gelu_tanh(g[r, j]) * f32(table[token[r], col0 + j])   (g f32 [rows][dim]; table bf16 [vocab][table_ld]; an id >= vocab reads row 0)
-uzu_status side_gate_mul(hipStream_t s, float* g, const uint32_t* tokens, const uint16_t* table, uint32_t table_ld, uint32_t col0, uint32_t vocab, uint32_t rows, uint32_t dim);
 
 // hidden[r * top + j, f] = act(gate_e x_r, up_e x_r) for e = ids[r, j] < routed; w13 bf16 [routed][2 ff][d], rows [0, ff) of an expert = up, [ff, 2 ff) = gate
 uzu_status moe_experts_gate_up(hipStream_t s, const float* x, const int32_t* ids, const uint16_t* w13, float* hidden, uint32_t rows, uint32_t d, uint32_t ff, uint32_t routed,

@@ -46,6 +46,7 @@ __global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tok
     for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) dst[i] = bf16_to_f32(src[i]) * scale; // (scale 1: the value itself)
 }
 
+constexpr int kNormUnroll = 8;
 // a workgroup per row: the sum of squares as 256 strided partial sums folded in a fixed tree, then the scaled row
 __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t d,
                                                             float offset) {
@@ -62,9 +63,23 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, floa
     }
     const float inv = 1.0f / sqrtf(s_red[0] / (float)d + eps);
     float* o = out + (size_t)r * d;
-    for (uint32_t i = threadIdx.x; i < d; i += 256) {
-        const float v = xr[i] * inv * gain;
-        o[i] = scales ? v * (scales[i] + offset) : v;
+    // kNormUnroll elements per thread and step, every load of a step in front of its stores (out may alias x for the compiler: a loop of load -> store pairs would
+    // pay one memory round trip per element, which is what a one-row decode step's launch consists of)
+    for (uint32_t i0 = threadIdx.x; i0 < d; i0 += 256 * kNormUnroll) {
+        float xv[kNormUnroll], sv[kNormUnroll];
+#pragma unroll
+        for (int u = 0; u < kNormUnroll; ++u) {
+            const uint32_t i = i0 + u * 256;
+            xv[u] = i < d ? xr[i] : 0.0f;
+            sv[u] = (i < d && scales) ? scales[i] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kNormUnroll; ++u) {
+            const uint32_t i = i0 + u * 256;
+            if (i >= d) break;
+            const float v = xv[u] * inv * gain;
+            o[i] = scales ? v * (sv[u] + offset) : v;
+        }
     }
 }
 
@@ -87,12 +102,24 @@ __global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, 
     const float* res = residual + (size_t)r * d;
     float* o = out + (size_t)r * d;
     float acc2 = 0.0f;
-    for (uint32_t i = threadIdx.x; i < d; i += 256) {
-        float v = yr[i] * inv * (scales[i] + offset);
-        if (layer_scale) v *= layer_scale[i];
-        v = res[i] + v;
-        o[i] = v;
-        acc2 = fmaf(v, v, acc2);
+    for (uint32_t i0 = threadIdx.x; i0 < d; i0 += 256 * kNormUnroll) { // (loads of a step in front of its stores, as in rms_norm_rows_kernel; sums in the same order)
+        float yv[kNormUnroll], rv[kNormUnroll], sv[kNormUnroll], lv[kNormUnroll];
+#pragma unroll
+        for (int u = 0; u < kNormUnroll; ++u) {
+            const uint32_t i = i0 + u * 256;
+            const bool ok = i < d;
+            yv[u] = ok ? yr[i] : 0.0f, rv[u] = ok ? res[i] : 0.0f, sv[u] = ok ? scales[i] : 0.0f, lv[u] = (ok && layer_scale) ? layer_scale[i] : 1.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kNormUnroll; ++u) {
+            const uint32_t i = i0 + u * 256;
+            if (i >= d) break;
+            float v = yv[u] * inv * (sv[u] + offset);
+            if (layer_scale) v *= lv[u];
+            v = rv[u] + v;
+            o[i] = v;
+            acc2 = fmaf(v, v, acc2);
+        }
     }
     if (!next) return;
     __syncthreads(); // s_red[0] has been read by everyone
@@ -104,7 +131,20 @@ __global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, 
     }
     const float inv2 = 1.0f / sqrtf(s_red[0] / (float)d + next_eps);
     float* nx = next + (size_t)r * d;
-    for (uint32_t i = threadIdx.x; i < d; i += 256) nx[i] = o[i] * inv2 * (next_scales[i] + next_offset); // (the thread's own stores)
+    for (uint32_t i0 = threadIdx.x; i0 < d; i0 += 256 * kNormUnroll) { // (o: the thread's own stores)
+        float ov[kNormUnroll], sv[kNormUnroll];
+#pragma unroll
+        for (int u = 0; u < kNormUnroll; ++u) {
+            const uint32_t i = i0 + u * 256;
+            ov[u] = i < d ? o[i] : 0.0f, sv[u] = i < d ? next_scales[i] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kNormUnroll; ++u) {
+            const uint32_t i = i0 + u * 256;
+            if (i >= d) break;
+            nx[i] = ov[u] * inv2 * (sv[u] + next_offset);
+        }
+    }
 }
 
 __device__ __forceinline__ float gelu_tanh_f32(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
@@ -174,9 +214,12 @@ __device__ __forceinline__ float apply_token_mul(float v, const LinearF32Params&
     return v * bf16_to_f32(p.mul_table[(size_t)t * p.mul_ld + p.mul_col0 + n]);
 }
 
+// thread = (row, hidden unit): a one-row decode step still spreads over ff / 256 workgroups
 __global__ void __launch_bounds__(256) gated_act_rows_kernel(const float* y1, float* hidden, uint32_t ff, ExpertAct act) {
-    const float* src = y1 + (size_t)blockIdx.x * 2 * ff;
-    for (uint32_t f = threadIdx.x; f < ff; f += blockDim.x) hidden[(size_t)blockIdx.x * ff + f] = expert_act(src[ff + f], src[f], act);
+    const uint32_t f = blockIdx.x * 256 + threadIdx.x, r = blockIdx.y;
+    if (f >= ff) return;
+    const float* src = y1 + (size_t)r * 2 * ff;
+    hidden[(size_t)r * ff + f] = expert_act(src[ff + f], src[f], act);
 }
 
 // ---- few rows: a wave per output column, RT rows per pass over the weights
@@ -525,7 +568,7 @@ uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residua
 uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act) {
     if (!rows || !ff) return UZU_OK;
     UZU_REQUIRE(y1 && hidden, "gated_act_rows: null argument");
-    return launch_check([&] { hipLaunchKernelGGL(gated_act_rows_kernel, dim3(rows), dim3(256), 0, s, y1, hidden, ff, act); }, "gated_act_rows");
+    return launch_check([&] { hipLaunchKernelGGL(gated_act_rows_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, s, y1, hidden, ff, act); }, "gated_act_rows");
 }
 
 uzu_status dyn_tanh_norm(hipStream_t s, const DynTanhParams& p) {

@@ -329,6 +329,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             k::LatentAttentionParams ap{};
             ap.qlat = S.qlat, ap.out = S.ctx, ap.caches = caches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans, ap.row_seq = S.d_row_seq;
             ap.rows = rows, ap.heads = H, ap.rank = kw, ap.window = h.sliding_window_size;
+            if (rd && rank % 4 == 0) ap.value_rank = rank; // the rotated columns score and carry no value
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd);
             ap.nseq = nseq;
             // decode-sized passes: spread a tile's key blocks over workgroups (a constant of the layer, so that a captured step stays valid as the context grows)

@@ -200,6 +200,10 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
     const uint8_t* cache = (const uint8_t*)p.caches[q];
+    // a cache row whose tail takes part in the scores only (value_rank < rank): the score product stops behind the row's last 16-column step, the weighted sum
+    // covers the value columns' 32-column blocks only
+    const uint32_t vr = p.value_rank ? p.value_rank : p.rank;
+    const uint32_t nsteps = (p.rank + 15) / 16, nbv = (vr + 31) / 32;
 
     const uint32_t kstep = SPLIT ? 32 * gridDim.y : 32;
     for (uint32_t kb = kmin + (SPLIT ? 32 * blockIdx.y : 0); kb <= kmax; kb += kstep) {
@@ -210,6 +214,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
             if (kk <= kmax && e0 < p.rank) val = *(const u32x4_v*)(cache + ((size_t)kk * p.rank + e0) * 2);
             *(u32x4_v*)(s_c + key * CP + e0 * 2) = val;
             const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+            if (e0 >= nbv * 32) continue; // columns outside the value blocks have no transposed copy
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 *(uint16_t*)(s_ct + (e0 + 2 * e) * TP + key * 2) = (uint16_t)(w[e] & 0xFFFFu);
@@ -223,8 +228,10 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
         for (int r = 0; r < 16; ++r) st[r] = 0.0f;
 #pragma unroll
         for (int s = 0; s < 2 * NB; ++s) {
-            const u32x4_t a = *(const u32x4_t*)(s_c + l32 * CP + (s * 16 + half * 8) * 2);
-            st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, qf[s]), st, 0, 0, 0);
+            if ((uint32_t)s < nsteps) { // (a predicate, not a break: the loop stays unrolled and qf / o statically indexed)
+                const u32x4_t a = *(const u32x4_t*)(s_c + l32 * CP + (s * 16 + half * 8) * 2);
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, qf[s]), st, 0, 0, 0);
+            }
         }
         float mx = -INFINITY;
 #pragma unroll
@@ -248,8 +255,9 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
         m_run = m_new;
 #pragma unroll
         for (int b = 0; b < NB; ++b)
+            if ((uint32_t)b < nbv)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[b][r] *= corr;
+                for (int r = 0; r < 16; ++r) o[b][r] *= corr;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             u32x4_t hi, lw;
@@ -264,11 +272,13 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
             hi = u32x4_t{hw[0], hw[1], hw[2], hw[3]}, lw = u32x4_t{lwv[0], lwv[1], lwv[2], lwv[3]};
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const uint8_t* cr = s_ct + (b * 32 + l32) * TP + (16 * s2 + 4 * half) * 2;
-                const u32x2_v c0 = *(const u32x2_v*)cr, c1 = *(const u32x2_v*)(cr + 16);
-                const u32x4_t cf{c0.x, c0.y, c1.x, c1.y};
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, hi), o[b], 0, 0, 0);
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, lw), o[b], 0, 0, 0);
+                if ((uint32_t)b < nbv) {
+                    const uint8_t* cr = s_ct + (b * 32 + l32) * TP + (16 * s2 + 4 * half) * 2;
+                    const u32x2_v c0 = *(const u32x2_v*)cr, c1 = *(const u32x2_v*)(cr + 16);
+                    const u32x4_t cf{c0.x, c0.y, c1.x, c1.y};
+                    o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, hi), o[b], 0, 0, 0);
+                    o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, lw), o[b], 0, 0, 0);
+                }
             }
         }
     }
@@ -277,9 +287,10 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
         float* ws = p.split_ws + (((size_t)(sp.row0 + row) * p.heads + head) * gridDim.y + blockIdx.y) * (RP + 4);
 #pragma unroll
         for (int b = 0; b < NB; ++b)
+            if ((uint32_t)b < nbv)
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4)
-                *(f32x4_v*)(ws + b * 32 + 8 * g4 + 4 * half) = f32x4_v{o[b][4 * g4], o[b][4 * g4 + 1], o[b][4 * g4 + 2], o[b][4 * g4 + 3]};
+                for (int g4 = 0; g4 < 4; ++g4)
+                    *(f32x4_v*)(ws + b * 32 + 8 * g4 + 4 * half) = f32x4_v{o[b][4 * g4], o[b][4 * g4 + 1], o[b][4 * g4 + 2], o[b][4 * g4 + 3]};
         if (half == 0) ws[RP] = m_run, ws[RP + 1] = l_run;
         return;
     }
@@ -290,13 +301,14 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(LatentAttent
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
             const uint32_t col = b * 32 + 8 * g4 + 4 * half;
-            if (col < p.rank) *(f32x4_v*)(out + col) = f32x4_v{o[b][4 * g4] * inv, o[b][4 * g4 + 1] * inv, o[b][4 * g4 + 2] * inv, o[b][4 * g4 + 3] * inv};
+            if (col < vr) *(f32x4_v*)(out + col) = f32x4_v{o[b][4 * g4] * inv, o[b][4 * g4 + 1] * inv, o[b][4 * g4 + 2] * inv, o[b][4 * g4 + 3] * inv};
         }
 }
 
 // a workgroup per item: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the splits (a split that saw no key has l = 0 and m = -1e30: weight 0).
 // The splits' weights are formed once (one thread per split, through LDS); the sums over the splits run in split order.
-__global__ void __launch_bounds__(256) latent_attention_merge_kernel(const float* ws, float* out, uint32_t items, uint32_t splits, uint32_t rank, uint32_t rp) {
+// (cols <= rank: the value columns; an item's row of `out` is rank wide)
+__global__ void __launch_bounds__(256) latent_attention_merge_kernel(const float* ws, float* out, uint32_t items, uint32_t splits, uint32_t rank, uint32_t rp, uint32_t cols) {
     __shared__ float s_w[64];
     __shared__ float s_inv;
     const uint32_t item = blockIdx.x, tid = threadIdx.x;
@@ -315,7 +327,7 @@ __global__ void __launch_bounds__(256) latent_attention_merge_kernel(const float
     }
     __syncthreads();
     const float inv = s_inv;
-    for (uint32_t e = tid; e < rank; e += blockDim.x) {
+    for (uint32_t e = tid; e < cols; e += blockDim.x) {
         float acc = 0.0f;
         for (uint32_t s = 0; s < splits; ++s) acc = fmaf(s_w[s], base[(size_t)s * (rp + 4) + e], acc);
         out[(size_t)item * rank + e] = acc * inv;
@@ -353,6 +365,7 @@ uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p) {
     if (!p.rows) return UZU_OK;
     UZU_REQUIRE(p.qlat && p.out && p.caches && p.spans && p.row_seq && p.heads && p.rank, "latent_attention: null argument");
     UZU_UNSUPPORTED(p.rank > kLatentMaxRank, "latent_attention: latent rank %u above %u", p.rank, kLatentMaxRank);
+    UZU_REQUIRE(p.value_rank <= p.rank && p.value_rank % 4 == 0, "latent_attention: value_rank is a multiple of 4 of at most rank");
     UZU_UNSUPPORTED(p.form == 2 && !latent_attention_tiled_supported(p), "latent_attention: the tiled form takes a bf16 cache, rank %% 8 == 0, rank <= 256");
     if (p.form != 1 && latent_attention_tiled_supported(p)) {
         static LdsLimit lim4, lim8, lim4s, lim8s;
@@ -370,7 +383,7 @@ uzu_status latent_attention(hipStream_t s, const LatentAttentionParams& p) {
                 UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL((latent_attention_mfma_kernel<8, true>), grid, dim3(256), lds, s, p); }, "latent_attention_mfma_split"));
             }
             const uint32_t items = p.rows * p.heads;
-            return launch_check([&] { hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(items), dim3(256), 0, s, p.split_ws, p.out, items, splits, p.rank, rp); },
+            return launch_check([&] { hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(items), dim3(256), 0, s, p.split_ws, p.out, items, splits, p.rank, rp, p.value_rank ? p.value_rank : p.rank); },
                                 "latent_attention_merge");
         }
         if (rp == 128) {

@@ -155,8 +155,11 @@ struct LatentAttentionParams {
     uint32_t rows, heads, rank, window;
     float scale;
     uint32_t form; // 0: chosen by shape; 1: the simple form (a wave per row and head, keys one after the other); 2: the tiled form
+    // != 0: only the first value_rank columns of a cache row are values -- the rest (a rotated key part) takes part in the scores alone, and the matching columns of
+    // `out` are left unwritten by the tiled form (a multiple of 4, at most rank); 0: the whole row
     uint32_t nseq;  // entries of `spans`
     uint32_t tiles; // sum over the sequences of ceil(count * heads / 128): the tiled form's workgroups (the caller knows the counts)
+    uint32_t value_rank;
     // tiled form, few rows over many keys (decode): `splits` > 1 workgroups share the key blocks of an item tile, partial sums go through split_ws
     // (latent_attention_split_ws_bytes(rows, heads, rank, splits) bytes) and a merge launch.  0 / null: one workgroup walks all keys of its tile.
     uint32_t splits;

@@ -144,6 +144,21 @@ uzu_status uzu_hip_s32_window_attention(uzu_hip_context* ctx, const float* q, co
                                         uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t vdim, uint32_t window, float scale, float soft_cap, uint32_t cache_bf16, uint32_t form);
 uzu_status uzu_hip_s32_retention(uzu_hip_context* ctx, const float* q, const float* k, const float* v, const float* decay, float* state_inout, float* out, uint32_t rows,
                                  uint32_t start, uint32_t heads, uint32_t dim, uint32_t vdim, uint32_t form);
+/*   rms_norm_add: out = residual + rms(y) (scales + offset) layer_scale, optionally with the norm of the new rows for the next sublayer.
+ *   rotate_normed: rotate with a per-head RMS norm of queries / keys in front of it.   latent_rope_append: RMS-normed latent + rotated shared key part into
+ *   cache_inout [(start + rows)][rank + rope_dim], every query head's rotated part into qlat_out's last rope_dim columns (interleaved or half-split pairs).
+ *   gated_lru: short causal convolution, block-diagonal gates (true f32), S <- a S + sqrt(1 - a^2) i u with a = exp(-rate r softplus(lambda)), out = S gelu(gate
+ *   branch); state and convolution window in and out; form 0 dispatch, 1 position by position, 2 in pieces of 32 rows. */
+uzu_status uzu_hip_s32_rms_norm_add(uzu_hip_context* ctx, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
+                                    uint32_t rows, uint32_t d, float* next_out, const float* next_scales, float next_offset, float next_eps);
+uzu_status uzu_hip_s32_rotate_normed(uzu_hip_context* ctx, float* qk_inout, const float* cosines, const float* sines, const float* q_norm, const float* k_norm, float norm_eps,
+                                     uint32_t rows, uint32_t start, uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t rope_dim);
+uzu_status uzu_hip_s32_latent_rope_append(uzu_hip_context* ctx, const float* x, const float* scales, float eps, const float* cosines, const float* sines, float* cache_inout,
+                                          float* qlat_out, uint32_t cache_bf16, uint32_t interleaved, uint32_t start, uint32_t rows, uint32_t heads, uint32_t q_width, uint32_t rank,
+                                          uint32_t rope_dim);
+uzu_status uzu_hip_s32_gated_lru(uzu_hip_context* ctx, const float* branches, const float* conv_w, const float* conv_b, const uint16_t* gate_w, const float* gate_b,
+                                 const float* lambda, float rate, float* state_inout, float* conv_state_inout, float* out, uint32_t rows, uint32_t start, uint32_t width,
+                                 uint32_t blocks, uint32_t taps, uint32_t form);
 /* 1: the full library.  0: the `stream32` flavor (make -C uzu_amd/csrc stream32 -> libuzu_hip_stream32.so), built without the fused decode kernels of the
  * bf16-stream models -- four minutes of compile time that a first use serving only an f32-stream design does not need; it refuses bf16-stream models at creation. */
 int uzu_hip_decode_kernels_present(void);

@@ -361,4 +361,151 @@ uzu_status uzu_hip_s32_retention(uzu_hip_context* ctx, const float* q, const flo
     return UZU_OK;
 }
 
+// Weight-vector RMS norm of a sublayer's result joined to the stream: out = residual + rms(y) (scales + offset) layer_scale (layer_scale optional), and with
+// next_out the norm of the new rows for the sublayer that follows (next_scales + next_offset, next_eps).  Host arrays [rows][d].
+uzu_status uzu_hip_s32_rms_norm_add(uzu_hip_context* ctx, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
+                                    uint32_t rows, uint32_t d, float* next_out, const float* next_scales, float next_offset, float next_eps) {
+    UZU_REQUIRE(ctx && y && residual && out && scales && (!next_out || next_scales), "s32_rms_norm_add: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    float *dy, *dr, *ds, *dl = nullptr, *dn = nullptr, *dns = nullptr;
+    UZU_PROPAGATE(S.up(y, (size_t)rows * d, &dy));
+    UZU_PROPAGATE(S.up(residual, (size_t)rows * d, &dr)); // in place, as the engine runs it behind a dense block
+    UZU_PROPAGATE(S.up(scales, d, &ds));
+    if (layer_scale) UZU_PROPAGATE(S.up(layer_scale, d, &dl));
+    if (next_out) {
+        UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * d, &dn));
+        UZU_PROPAGATE(S.up(next_scales, d, &dns));
+    }
+    UZU_PROPAGATE(k::rms_norm_add_rows(ctx->stream, dy, dr, dr, ds, offset, dl, eps, rows, d, dn, dns, next_offset, next_eps));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dr, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
+    if (next_out) UZU_HIP_TRY(hipMemcpy(next_out, dn, (size_t)rows * d * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// uzu_hip_s32_rotate with a per-head RMS norm of queries (q_norm [dim] or NULL) and keys (k_norm) in front of the rotation
+uzu_status uzu_hip_s32_rotate_normed(uzu_hip_context* ctx, float* qk_inout, const float* cosines, const float* sines, const float* q_norm, const float* k_norm, float norm_eps,
+                                     uint32_t rows, uint32_t start, uint32_t heads, uint32_t kv_heads, uint32_t dim, uint32_t rope_dim) {
+    UZU_REQUIRE(ctx && qk_inout && (!rope_dim || (cosines && sines)), "s32_rotate_normed: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const uint32_t ld = (heads + kv_heads) * dim;
+    float *dx, *dc = nullptr, *ds = nullptr, *dqn = nullptr, *dkn = nullptr;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up((const float*)qk_inout, (size_t)rows * ld, &dx));
+    if (rope_dim) {
+        UZU_PROPAGATE(S.up(cosines, (size_t)(start + rows) * rope_dim, &dc));
+        UZU_PROPAGATE(S.up(sines, (size_t)(start + rows) * rope_dim, &ds));
+    }
+    if (q_norm) UZU_PROPAGATE(S.up(q_norm, dim, &dqn));
+    if (k_norm) UZU_PROPAGATE(S.up(k_norm, dim, &dkn));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::RopeAppendParams p{};
+    p.qkv = dx, p.ld = ld, p.k_col = heads * dim, p.v_col = ld, p.heads = heads, p.kv_heads = kv_heads, p.dim = dim, p.vdim = 0, p.rope_dim = rope_dim, p.cosines = dc, p.sines = ds;
+    p.key_scale = 1.0f, p.q_norm = dqn, p.k_norm = dkn, p.norm_eps = norm_eps, p.spans = spans, p.row_seq = row_seq, p.rows = rows;
+    UZU_PROPAGATE(k::rope_append(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(qk_inout, dx, (size_t)rows * ld * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// x [rows][heads * q_width + rank + rope_dim]: query heads (the last rope_dim coordinates of each turn), then the down projection's row.  cache_inout
+// [(start + rows)][rank + rope_dim] f32 (rows below `start` come back as given); qlat_out [rows][heads][rank + rope_dim]: only the rotated columns are written
+// (the others come back as NaN).  Tables [start + rows][rope_dim].
+uzu_status uzu_hip_s32_latent_rope_append(uzu_hip_context* ctx, const float* x, const float* scales, float eps, const float* cosines, const float* sines, float* cache_inout,
+                                          float* qlat_out, uint32_t cache_bf16, uint32_t interleaved, uint32_t start, uint32_t rows, uint32_t heads, uint32_t q_width, uint32_t rank,
+                                          uint32_t rope_dim) {
+    UZU_REQUIRE(ctx && x && scales && cache_inout && qlat_out && (!rope_dim || (cosines && sines)), "s32_latent_rope_append: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const uint32_t kw = rank + rope_dim, ldx = heads * q_width + kw;
+    const size_t total = (size_t)(start + rows) * kw;
+    float *dx, *dsc, *dc = nullptr, *dsn = nullptr, *dc32 = nullptr, *dq;
+    uint16_t* dc16 = nullptr;
+    void** dcp;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up(x, (size_t)rows * ldx, &dx));
+    UZU_PROPAGATE(S.up(scales, rank, &dsc));
+    if (rope_dim) {
+        UZU_PROPAGATE(S.up(cosines, (size_t)(start + rows) * rope_dim, &dc));
+        UZU_PROPAGATE(S.up(sines, (size_t)(start + rows) * rope_dim, &dsn));
+    }
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * heads * kw, &dq));
+    std::vector<uint16_t> bits(total);
+    if (cache_bf16) {
+        for (size_t i = 0; i < total; ++i) bits[i] = f32_to_bf16(cache_inout[i]);
+        UZU_PROPAGATE(S.up(bits.data(), total, &dc16));
+    } else {
+        UZU_PROPAGATE(S.up((const float*)cache_inout, total, &dc32));
+    }
+    void* cache = cache_bf16 ? (void*)dc16 : (void*)dc32;
+    UZU_PROPAGATE(S.up((void* const*)&cache, 1, &dcp));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::LatentRopeAppendParams p{};
+    p.x = dx, p.ldx = ldx, p.c_col = heads * q_width, p.rank = rank, p.rope_dim = rope_dim, p.scales = dsc, p.eps = eps, p.caches = dcp, p.cache_bf16 = cache_bf16, p.heads = heads;
+    p.q_width = q_width, p.qlat = rope_dim ? dq : nullptr, p.cosines = dc, p.sines = dsn, p.interleaved = interleaved, p.spans = spans, p.row_seq = row_seq, p.rows = rows;
+    UZU_PROPAGATE(k::latent_rope_append(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    if (cache_bf16) {
+        UZU_HIP_TRY(hipMemcpy(bits.data(), dc16, total * 2, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < total; ++i) cache_inout[i] = bf16_to_f32(bits[i]);
+    } else {
+        UZU_HIP_TRY(hipMemcpy(cache_inout, dc32, total * 4, hipMemcpyDeviceToHost));
+    }
+    UZU_HIP_TRY(hipMemcpy(qlat_out, dq, (size_t)rows * heads * kw * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
+// The gated linear recurrent unit on rows at positions start ..: branches [rows][2 width] (gate branch | recurrent branch, biases added), conv_w [width][taps],
+// conv_b [width], gate_w bf16 [blocks][2 bw][bw], gate_b [blocks][2 bw], lambda [width]; state_inout [width] and conv_state_inout [taps - 1][width] (at least one
+// row) are the state in front of the rows (ignored where positions lie in front of 0) and behind them; out [rows][width] = S * gelu(gate branch).
+// form 0 dispatch, 1 position by position, 2 in pieces.
+uzu_status uzu_hip_s32_gated_lru(uzu_hip_context* ctx, const float* branches, const float* conv_w, const float* conv_b, const uint16_t* gate_w, const float* gate_b,
+                                 const float* lambda, float rate, float* state_inout, float* conv_state_inout, float* out, uint32_t rows, uint32_t start, uint32_t width,
+                                 uint32_t blocks, uint32_t taps, uint32_t form) {
+    UZU_REQUIRE(ctx && branches && conv_w && gate_w && lambda && state_inout && conv_state_inout && out && blocks && width % blocks == 0 && taps, "s32_gated_lru: null argument");
+    (void)hipSetDevice(ctx->device);
+    Scratch S;
+    const uint32_t bw = width / blocks, keep = taps > 1 ? taps - 1 : 1;
+    float *dx, *dcw, *dcb = nullptr, *dgb = nullptr, *dl, *dst, *dcs, *du, *dg, *dout, *dws;
+    uint16_t* dgw;
+    float **dsp, **dcsp;
+    k::SeqSpan* spans;
+    uint32_t* row_seq;
+    UZU_PROPAGATE(S.up(branches, (size_t)rows * 2 * width, &dx));
+    UZU_PROPAGATE(S.up(conv_w, (size_t)width * taps, &dcw));
+    if (conv_b) UZU_PROPAGATE(S.up(conv_b, width, &dcb));
+    UZU_PROPAGATE(S.up(gate_w, (size_t)2 * width * bw, &dgw));
+    if (gate_b) UZU_PROPAGATE(S.up(gate_b, (size_t)2 * width, &dgb));
+    UZU_PROPAGATE(S.up(lambda, width, &dl));
+    UZU_PROPAGATE(S.up((const float*)state_inout, width, &dst));
+    UZU_PROPAGATE(S.up((const float*)conv_state_inout, (size_t)keep * width, &dcs));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * width, &du));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * 2 * width, &dg));
+    UZU_PROPAGATE(S.up((const float*)nullptr, (size_t)rows * width, &dout));
+    UZU_PROPAGATE(S.up((float* const*)&dst, 1, &dsp));
+    UZU_PROPAGATE(S.up((float* const*)&dcs, 1, &dcsp));
+    UZU_PROPAGATE(one_sequence(S, rows, start, &spans, &row_seq));
+    k::GatedLruParams p{};
+    p.branches = dx, p.ld = 2 * width, p.x_col = width, p.u = du, p.gates = dg, p.out = dout, p.conv_w = dcw, p.conv_b = dcb, p.gate_b = dgb, p.lambda = dl, p.rate = rate;
+    p.states = dsp, p.conv_states = dcsp, p.spans = spans, p.row_seq = row_seq, p.nseq = 1, p.rows = rows, p.width = width, p.blocks = blocks, p.taps = taps, p.form = form;
+    p.max_count = rows, p.pieces = (rows + 31) / 32, p.piece_ws_bytes = k::lru_piece_ws_bytes(p.pieces, width);
+    UZU_PROPAGATE(S.up((const float*)nullptr, p.piece_ws_bytes / 4, &dws));
+    p.piece_ws = dws;
+    UZU_PROPAGATE(k::lru_conv(ctx->stream, p));
+    k::LinearF32Params g{};
+    g.x = du, g.w = dgw, g.y = dg, g.rows = rows, g.n = 2 * bw, g.k = bw, g.ldx = width, g.ldy = 2 * width, g.batch = blocks, g.x_batch = bw, g.w_batch = (size_t)2 * bw * bw;
+    g.y_batch = 2 * bw, g.bf16_products = 0;
+    UZU_PROPAGATE(k::linear_f32(ctx->stream, g));
+    UZU_PROPAGATE(k::lru_scan(ctx->stream, p));
+    UZU_PROPAGATE(finish(ctx));
+    UZU_HIP_TRY(hipMemcpy(out, dout, (size_t)rows * width * 4, hipMemcpyDeviceToHost));
+    UZU_HIP_TRY(hipMemcpy(state_inout, dst, (size_t)width * 4, hipMemcpyDeviceToHost));
+    UZU_HIP_TRY(hipMemcpy(conv_state_inout, dcs, (size_t)keep * width * 4, hipMemcpyDeviceToHost));
+    return UZU_OK;
+}
+
 } // extern "C"

@@ -405,3 +405,59 @@ def test_refusals_of_the_engine(hip_ctx, tmp_path):
     bf16 = dataclasses.replace(bundle, f32_stream=False)
     with pytest.raises(_ffi.UzuHipError):
         HipModel(hip_ctx, bf16, 0)
+
+
+def random_config(seed):
+    """a configuration drawn at random: sizes, head counts, layer order, loop, constants"""
+    rng = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(rng.integers(len(xs)))]
+    width = pick(24, 40, 64, 96, 136)
+    scaling = lambda: pick(None, {"factor": pick(2.0, 4.0, 8.0), "original": pick(16, 64, 256), "fast": pick(8.0, 32.0), "slow": pick(1.0, 2.0)})
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        mlp = pick(None, O.dense(pick(16, 40, 72), pick(0.5, 1.0, 7.0)))
+        kind = pick("latent", "attention", "rglru")
+        if kind == "latent":
+            rd = pick(2, 4, 8, 16)
+            layers.append(O.latent_layer(pick(1, 2, 4, 6), pick(4, 8, 16, 24), rd, pick(4, 12, 16, 40), pick(8, 24, 56, 120), O.rot(rd, pick(1e3, 1e4, 5e5), scaling()),
+                                         scale=pick(0.1, 0.2, 0.35), mlp=mlp))
+        elif kind == "attention":
+            G = pick(1, 2, 3)
+            dim = pick(8, 16, 32, 64)
+            layers.append(O.attention_layer(G * pick(1, 2, 4), G, dim, pick(8, 16, 24), O.rot(pick(0, 2, dim // 2, dim), pick(1e3, 1e4, 5e4), scaling()), scale=pick(0.1, 0.2, 0.35), mlp=mlp))
+        else:
+            blocks = pick(1, 2, 4, 5)
+            layers.append(O.rglru_layer(blocks * pick(4, 8, 20), blocks, pick(1, 2, 3, 4), mlp=mlp))
+    n = len(layers)
+    loop = None
+    if rng.random() < 0.8:
+        a = int(rng.integers(0, n))
+        loop = (a, int(rng.integers(a + 1, n + 1)), pick(1, 2, 3))
+    return O.config(vocab=pick(50, 257, 640), width=width, layers=layers, eps=pick(1e-6, 1e-5, 1e-3), embed_scale=pick(1.0, 4.0, 12.0), logit_scale=pick(0.25, 1.0, 3.0), loop=loop,
+                    side_dim=pick(0, 3, 8, 24))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(hip_ctx, tmp_path, seed):
+    """whole prompt, prompt + decoded tail and an unequal batch on a configuration nobody chose, in both precisions"""
+    cfg = random_config(100 + seed)
+    W = O.weights(cfg, seed)
+    O.write_model_dir(str(tmp_path / "m"), cfg, W)
+    W64 = {k: v.astype(np.float64) for k, v in W.items()}
+    bundle = loader.load_model_dir(str(tmp_path / "m"), max_context_length=400)
+    a, b = prompt(cfg, 170, seed), prompt(cfg, 45, seed + 50)
+    want_a, want_b = O.forward(cfg, W64, a)[0], O.forward(cfg, W64, b)[0]
+    for full in (True, False):
+        m = HipModel(hip_ctx, bundle, MODEL_BATCH(3) | (MODEL_FULL_F32 if full else 0))
+        st = m.new_state()
+        whole, _ = m.step_batch([st], [a], [list(range(170))])
+        st.reset()
+        head, _ = m.step_batch([st], [a[:130]], [list(range(130))])
+        tail = [m.step_batch([st], [[t]], [[0]])[0][0] for t in a[130:]]
+        st2 = m.new_state()
+        st.reset()
+        both, _ = m.step_batch([st2, st], [b, a[:100]], [list(range(45)), list(range(100))])
+        for got, want in ((whole, want_a), (np.concatenate([head, np.stack(tail)]), want_a), (both[:45], want_b), (both[45:], want_a[:100])):
+            err = O.logit_error(got, want)
+            assert (err.max() < TOL[True]) if full else (np.median(err) < 3e-2 and np.mean(err < 8e-2) >= 0.9), (cfg, full, err.max(), np.median(err))
+        m.close()

@@ -93,7 +93,8 @@ typedef struct {
     const float* scales;    /* f32 [dim] or NULL (has_scale == false) */
     const float* biases;    /* f32 [dim] or NULL */
     float alpha;            /* UZU_NORM_DYNAMIC_TANH: the scalar inside the tanh; UZU_NORM_RMS_SCALAR: the gain */
-    uint32_t reserved;
+    uint32_t groups;        /* f32-stream designs, UZU_NORM_STATISTICS: the row is cut into `groups` equal consecutive parts, each divided by its own root mean
+                               square (dim % groups == 0); 0 or 1 = the whole row (the field was `reserved`) */
 } uzu_norm_desc;
 
 typedef enum {
@@ -310,6 +311,41 @@ typedef struct {
     uint32_t weights_of_layer;
     /* Re-entry of the stream: before this run x <- W [x ; x0] with x0 the embedding rows (n = model_dim, k = 2 model_dim); absent = none */
     uzu_linear_desc stream_reentry;
+    /* Input convolution of the sublayers (f32-stream designs): what a sublayer reads is h + conv(h), h = its input rows (the stream itself where the pre norm is
+     * absent -- with an input convolution pre_mixer_norm / pre_mlp_norm may be absent), conv = a causal convolution over positions on every channel:
+     * conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j), zeros in front of the sequence; input_conv_mixer / input_conv_mlp f32 [model_dim, input_conv_taps] (either
+     * may be NULL = that sublayer reads h).  The last taps - 1 inputs of each are sequence state. */
+    uint32_t input_conv_taps;
+    /* UZU_MIXER_ATTENTION in an f32-stream design, further options: */
+    uint32_t qk_norm_whole;        /* query_norm / key_norm are ONE RMS norm over the whole projection each (scales [heads head_dim] / [groups head_dim]), not per head */
+    const float* input_conv_mixer;
+    const float* input_conv_mlp;
+    uint32_t attention_chunk_size; /* != 0: position i sees j <= i only inside its own chunk, floor(i / size) == floor(j / size), chunks counted from position 0 */
+    uint32_t values_are_keys;      /* the packed projection has no value rows: the values are the key rows as projected (before their norm and rotation);
+                                      value_head_dim == head_dim */
+    uint32_t rel_bias_rows;        /* != 0: a learned bias per (distance bucket, head) is added to the scaled score: rel_bias bf16 [rel_bias_rows, heads]; with
+                                      E = rows / 2 the bucket of distance n is n below E, else min(rows - 1, E + floor(ln(n / E) / ln(rel_bias_max / E) (rows - E))) */
+    float rel_bias_max;
+    const uint16_t* rel_bias;
+    const float* head_temperature; /* f32 [heads] or NULL: the scaled score of head a is multiplied by head_temperature[a] (in front of the bias) */
+    /* has_gate on such a layer: num_heads more rows behind the packed projection's values; head a's result is multiplied by sigmoid(row a . h). */
+    /* A second mixer beside the first (f32-stream designs): both read the same rows, the layer's mixer result is pair_scale_main * main + pair_scale_second *
+     * second, each through its own out projection.  pair_mixer = 1 + uzu_mixer_kind of the second (0 = none); supported: attention with a channel-decay delta
+     * rule (UZU_MIXER_DELTA_NET) as the second. */
+    uint32_t pair_mixer;
+    float pair_scale_main, pair_scale_second;
+    /* UZU_MIXER_DELTA_NET in an f32-stream design: the gated delta rule with one decay per head and KEY CHANNEL.  dn_num_heads value heads of dn_value_head_dim on
+     * dn_num_groups query / key heads of dn_head_dim (head a reads group a / (heads / groups)).  dn_in_proj rows: q | k | v | beta (heads) | decay down
+     * (dn_decay_rank) | gate down (dn_gate_rank); q, k, v pass a causal convolution per channel (dn_kernel_size taps, dn_conv_weights f32 [2 groups dk + heads dv,
+     * taps], no bias) and silu; q and k become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q times dk^(-1/2); beta = sigmoid; decay[a, c] =
+     * exp(-exp(dn_a_log[a]) softplus(dn_decay_up (decay down) + dn_dt_bias))[a dk + c] (dn_dt_bias f32 [heads dk]); per head S <- decay * S (rows = key
+     * channels), u = beta (v - S^T k), S <- S + k u^T, o = S^T q; o / rms(o over dv, dn_norm_epsilon) * dn_norm_scales * sigmoid(dn_gate_up (gate down)); then
+     * dn_out_proj.  S (f32 [heads, dk, dv], zero in front of position 0) and the convolution's last taps - 1 inputs are sequence state.  Everything behind the
+     * projections and the convolution is f32 in both precisions, the two up products included. */
+    uint32_t dn_channel_decay;
+    uint32_t dn_decay_rank, dn_gate_rank;
+    uzu_linear_desc dn_decay_up; /* n = heads dk, k = dn_decay_rank */
+    uzu_linear_desc dn_gate_up;  /* n = heads dv, k = dn_gate_rank */
 } uzu_layer_desc;
 
 typedef struct {
@@ -351,7 +387,12 @@ typedef struct {
      * tied embedding table behind output_norm; logits are f32.  Such a model runs through its own forward encoder (csrc/engine_stream32.hip), batched over
      * sequences of unequal length (uzu_hip_model_step_batch). */
     uint32_t f32_stream;
-    uint32_t reserved5;
+    /* A second, hashed token table added to the looked-up rows (f32-stream designs): row (previous token * bigram_mul_prev + token * bigram_mul_cur) mod
+     * bigram_buckets of bigram_table (bf16 [bigram_buckets + 1, model_dim], not scaled by input_scale); a sequence's first token reads the last row.  The previous
+     * token is sequence state.  bigram_buckets == 0: none (the field was `reserved5`). */
+    uint32_t bigram_buckets;
+    uint32_t bigram_mul_prev, bigram_mul_cur;
+    uzu_linear_desc bigram_table;
 } uzu_model_desc;
 
 /*

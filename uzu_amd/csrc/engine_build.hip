@@ -129,6 +129,7 @@ uzu_status state_build(uzu_hip_model* m, uzu_hip_state** out) {
     need((size_t)m->chunk * 4, &p), st->d_tokens = (uint32_t*)p;
     need(4, &p), st->d_out_token = (uint32_t*)p;
     need((size_t)m->max_positions * 4, &p), st->d_sampled = (uint32_t*)p;
+    if (m->d.bigram_buckets) need(4, &p), st->prev_token = (uint32_t*)p; // (read only behind position 0)
     if (r != UZU_OK) {
         state_free(st);
         return r;
@@ -240,6 +241,7 @@ uzu_status upload_linear(uzu_hip_model* m, const uzu_linear_desc& h, DLinear* o,
 uzu_status upload_norm(uzu_hip_model* m, const uzu_norm_desc& h, uint32_t dim, DNorm* o) {
     o->present = h.present != 0;
     o->full_layer = h.full_layer, o->subtract_mean = h.subtract_mean, o->eps = h.epsilon, o->offset = h.scale_offset;
+    o->groups = h.groups ? h.groups : 1;
     if (!o->present) return UZU_OK;
     UZU_PROPAGATE(upload(m, h.scales, (size_t)dim * 4, &o->scales));
     UZU_PROPAGATE(upload(m, h.biases, (size_t)dim * 4, &o->biases));
@@ -336,8 +338,11 @@ uzu_status uzu_hip_model_create_tp(uzu_hip_context* ctx, const uzu_model_desc* d
                         (desc->layers[l].mlp_kind == UZU_MLP_MOE && desc->layers[l].moe.routing != UZU_MOE_ROUTE_TOPK_LOGITS) ||
                         desc->layers[l].mixer_kind == UZU_MIXER_GATED_LRU || desc->layers[l].latent_rope_dim || desc->layers[l].latent_packed || desc->layers[l].rope_interleaved ||
                         desc->layers[l].layer_scale_mixer || desc->layers[l].layer_scale_mlp || desc->layers[l].weights_of_layer || desc->layers[l].stream_reentry.weights ||
-                        desc->layers[l].ple_slice,
+                        desc->layers[l].ple_slice || desc->layers[l].input_conv_taps || desc->layers[l].qk_norm_whole || desc->layers[l].attention_chunk_size ||
+                        desc->layers[l].values_are_keys || desc->layers[l].rel_bias_rows || desc->layers[l].head_temperature || desc->layers[l].pair_mixer ||
+                        desc->layers[l].dn_channel_decay || desc->layers[l].post_mixer_norm.groups > 1 || desc->layers[l].post_mlp_norm.groups > 1,
                         "model_create: layer %u uses a mechanism of the f32-stream designs (set uzu_model_desc::f32_stream)", l);
+    UZU_UNSUPPORTED(desc->bigram_buckets || desc->output_norm.groups > 1, "model_create: a hashed token-pair table and grouped norms are mechanisms of the f32-stream designs");
     (void)hipSetDevice(ctx->device);
     auto* m = new uzu_hip_model();
     m->ctx = ctx;

@@ -52,6 +52,12 @@ struct Stream32 {
     void** d_cache_ptrs = nullptr;  // [layers][max_seqs]: latent rows / key rows / the retention state
     void** d_cache2_ptrs = nullptr; // [layers][max_seqs]: value rows
     float** d_shift_ptrs = nullptr; // [layers][max_seqs]
+    float** d_pair_state_ptrs = nullptr; // [layers][max_seqs]: the second mixer's recurrent state
+    float** d_pair_conv_ptrs = nullptr;  // [layers][max_seqs]: ... and its convolution window
+    float** d_inconv_ptrs = nullptr;     // [layers][max_seqs]: the windows of the sublayers' input convolutions (mixer's, then MLP's)
+    uint32_t** d_prev_tok_ptrs = nullptr; // [max_seqs]: the previous token (hashed token-pair table)
+    float *dn_in = nullptr, *dn_cv = nullptr, *dn_decay = nullptr, *dn_gate = nullptr, *dn_o = nullptr; // the delta rule: packed projection, convolved q | k | v, decays, gate, result
+    uint16_t* pair_table = nullptr; // bf16 [buckets + 1][d]
     struct Layer {
         uint16_t* up_keys_t = nullptr; // bf16 [heads][rank][head_dim]: W_up_k of a head transposed, so that folding it into the query is an ordinary product
         float* sinks = nullptr;        // f32 [heads]
@@ -62,6 +68,11 @@ struct Stream32 {
         uint16_t* lru_gate_w = nullptr;       // gated LRU: bf16 [blocks][2 bw][bw]
         float *lru_gate_b = nullptr, *lru_lambda = nullptr;
         DLinear reentry_a, reentry_b; // the re-entry projection's halves: on the stream, on the embedding rows
+        float *in_conv_mixer = nullptr, *in_conv_mlp = nullptr; // input convolutions f32 [d][taps]
+        float* dist_bias = nullptr;   // f32 [dist_rows][heads]: the distance bias by distance (the bucket rule applied on the host)
+        uint32_t dist_rows = 0;
+        float* head_temp = nullptr;   // f32 [heads]
+        DLinear decay_up, gate_up;    // the delta rule's low-rank second factors
     };
     std::vector<Layer> layers;
     float alpha_out = 0.f;
@@ -131,7 +142,7 @@ void run_norm(Enc& e, const DNorm& N, uint32_t kind, float alpha, const float* x
         return;
     }
     if (kind == UZU_NORM_STATISTICS) { // RMS with a weight vector (+ offset)
-        RUN("rms_norm_rows", (size_t)rows * d * 8, k::rms_norm_rows(s, x, out, N.scales, 1.0f, N.eps, row_index, rows, d, N.offset));
+        RUN("rms_norm_rows", (size_t)rows * d * 8, k::rms_norm_rows(s, x, out, N.scales, 1.0f, N.eps, row_index, rows, d, N.offset, N.groups));
         return;
     }
     k::DynTanhParams np{};
@@ -165,7 +176,10 @@ uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs,
     }
     UZU_REQUIRE(rows <= S.max_rows, "engine: a pass of %u rows (at most %u)", rows, S.max_rows);
     std::vector<void*> cache_ptrs((size_t)nl * S.max_seqs, nullptr), cache2_ptrs((size_t)nl * S.max_seqs, nullptr);
-    std::vector<float*> shift_ptrs((size_t)nl * S.max_seqs, nullptr);
+    std::vector<float*> shift_ptrs((size_t)nl * S.max_seqs, nullptr), pair_state((size_t)nl * S.max_seqs, nullptr), pair_conv((size_t)nl * S.max_seqs, nullptr);
+    std::vector<float*> inconv((size_t)nl * S.max_seqs, nullptr);
+    std::vector<uint32_t*> prev_tok(S.max_seqs, nullptr);
+    for (uint32_t i = 0; i < nseq; ++i) prev_tok[i] = seqs[i].st->prev_token;
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = m->layers[l].d;
         const uint32_t src = h.is_kv_sharing ? h.kv_source_layer_index : l;
@@ -177,6 +191,8 @@ uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs,
             else if (h.mixer_kind == UZU_MIXER_RETENTION) cache_ptrs[at] = own.ret_state;
             else cache_ptrs[at] = own.latent;
             shift_ptrs[at] = seqs[i].st->layers[l].shift_prev;
+            inconv[at] = seqs[i].st->layers[l].in_conv;
+            if (h.pair_mixer) pair_state[at] = seqs[i].st->layers[l].ssm_state, pair_conv[at] = seqs[i].st->layers[l].conv_state;
         }
     }
     // (pageable sources: the copies have left the host buffers when the calls return)
@@ -185,6 +201,12 @@ uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs,
     HIPCHK(hipMemcpyAsync(S.d_cache_ptrs, cache_ptrs.data(), cache_ptrs.size() * sizeof(void*), hipMemcpyHostToDevice, s));
     HIPCHK(hipMemcpyAsync(S.d_cache2_ptrs, cache2_ptrs.data(), cache2_ptrs.size() * sizeof(void*), hipMemcpyHostToDevice, s));
     HIPCHK(hipMemcpyAsync(S.d_shift_ptrs, shift_ptrs.data(), shift_ptrs.size() * sizeof(float*), hipMemcpyHostToDevice, s));
+    if (S.d_pair_state_ptrs) {
+        HIPCHK(hipMemcpyAsync(S.d_pair_state_ptrs, pair_state.data(), pair_state.size() * sizeof(float*), hipMemcpyHostToDevice, s));
+        HIPCHK(hipMemcpyAsync(S.d_pair_conv_ptrs, pair_conv.data(), pair_conv.size() * sizeof(float*), hipMemcpyHostToDevice, s));
+    }
+    if (S.d_inconv_ptrs) HIPCHK(hipMemcpyAsync(S.d_inconv_ptrs, inconv.data(), inconv.size() * sizeof(float*), hipMemcpyHostToDevice, s));
+    if (S.d_prev_tok_ptrs) HIPCHK(hipMemcpyAsync(S.d_prev_tok_ptrs, prev_tok.data(), prev_tok.size() * sizeof(uint32_t*), hipMemcpyHostToDevice, s));
     if (!out_rows.empty()) HIPCHK(hipMemcpyAsync(S.d_out_rows, out_rows.data(), out_rows.size() * 4, hipMemcpyHostToDevice, s));
     return UZU_OK;
 }
@@ -203,7 +225,16 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     for (uint32_t c : counts) rows += c;
     const size_t slot_stride = (size_t)S.max_rows * d;
     const uint32_t bf = S.full_f32 ? 0u : 1u;
-    RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d, m->d.input_scale));
+    if (S.pair_table) { // + the hashed (previous token, token) row; two launches: the rows, then the sequences' new previous tokens
+        k::EmbedPairParams ep{};
+        ep.tokens = d_tokens, ep.table = (const uint16_t*)m->embedding.w, ep.pair_table = S.pair_table, ep.out = S.slots, ep.rows = rows, ep.vocab = m->d.vocab_size, ep.d = d;
+        ep.scale = m->d.input_scale, ep.buckets = m->d.bigram_buckets, ep.mul_prev = m->d.bigram_mul_prev, ep.mul_cur = m->d.bigram_mul_cur, ep.spans = S.d_spans;
+        ep.row_seq = S.d_row_seq, ep.prev = S.d_prev_tok_ptrs, ep.nseq = nseq;
+        RUN("embed_pair_rows_f32", (size_t)rows * d * 8, k::embed_pair_rows_f32(s, ep));
+        ++m->launches;
+    } else {
+        RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d, m->d.input_scale));
+    }
     const float* cur = S.slots; // what the layer about to run reads: X_0, then the depth mix of the layer before
     uint32_t max_count = 0;
     for (uint32_t c : counts) max_count = std::max(max_count, c);
@@ -212,7 +243,18 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     auto add_normed = [&](const float* y, const float* residual, float* out, const DNorm& N, const float* layer_scale, const DNorm* next) {
         RUN("rms_norm_add_rows", (size_t)rows * d * (next ? 16 : 12),
             k::rms_norm_add_rows(s, y, residual, out, N.scales, N.offset, layer_scale, N.eps, rows, d, next ? S.normed : nullptr, next ? next->scales : nullptr,
-                                 next ? next->offset : 0.0f, next ? next->eps : 0.0f));
+                                 next ? next->offset : 0.0f, next ? next->eps : 0.0f, N.groups));
+    };
+    // what a sublayer without a pre norm reads: the stream rows themselves, or (with an input convolution) rows + conv(rows) in S.normed; `which` = 0 the mixer's
+    // window of the layer's state, 1 the MLP's.  The window is replaced right away: `x` still holds the pass's inputs here.
+    auto conv_input = [&](uint32_t l, const float* x, const float* w, uint32_t taps, uint32_t which) -> const float* {
+        if (!w) return x;
+        k::CausalConvParams cp{};
+        cp.x = x, cp.ldx = d, cp.out = S.normed, cp.ldo = d, cp.w = w, cp.channels = d, cp.taps = taps, cp.add_input = 1;
+        cp.states = S.d_inconv_ptrs + (size_t)l * S.max_seqs, cp.state_offset = (size_t)which * (taps - 1) * d, cp.spans = S.d_spans, cp.row_seq = S.d_row_seq, cp.nseq = nseq, cp.rows = rows;
+        RUN("causal_conv_rows", (size_t)rows * d * 4 * (taps + 1), k::causal_conv_rows(s, cp));
+        if (taps > 1) RUN("causal_conv_commit", (size_t)nseq * d * 8 * (taps - 1), k::causal_conv_commit(s, cp));
+        return S.normed;
     };
     bool normed_ready = false; // S.normed already holds this run's pre-mixer norm (left by the run before)
     for (uint32_t l = 0; l < nl; ++l) {
@@ -230,11 +272,18 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         }
         // which launch ends this run, and whether it can leave the next run's pre-mixer norm
         const DNorm* next_pre = nullptr;
-        if (l + 1 < nl && !X.depth_weights && !S.layers[l + 1].reentry_a.w && m->layers[l + 1].d.pre_mixer_norm.kind == UZU_NORM_STATISTICS) next_pre = &m->layers[l + 1].pre_mixer;
-        const bool pre_mlp_fused = !h.no_mlp && !h.parallel_block && L.post_mixer.present && h.pre_mlp_norm.kind == UZU_NORM_STATISTICS;
+        if (l + 1 < nl && !X.depth_weights && !S.layers[l + 1].reentry_a.w && m->layers[l + 1].pre_mixer.present && m->layers[l + 1].d.pre_mixer_norm.kind == UZU_NORM_STATISTICS &&
+            m->layers[l + 1].pre_mixer.groups <= 1)
+            next_pre = &m->layers[l + 1].pre_mixer;
+        const bool pre_mlp_fused = !h.no_mlp && !h.parallel_block && L.post_mixer.present && L.post_mixer.groups <= 1 && L.pre_mlp.present && h.pre_mlp_norm.kind == UZU_NORM_STATISTICS &&
+                                   L.pre_mlp.groups <= 1;
+        if (next_pre && ((L.post_mixer.present && L.post_mixer.groups > 1) || (L.post_mlp.present && L.post_mlp.groups > 1) || (h.has_ple && L.ple_norm.groups > 1))) next_pre = nullptr;
         const bool have_normed = normed_ready;
         normed_ready = false;
+        const float* mix_in = S.normed; // the rows the mixer reads
         if (have_normed) {
+        } else if (!L.pre_mixer.present) {
+            mix_in = conv_input(l, cur, X.in_conv_mixer, h.input_conv_taps, 0);
         } else if (h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH) {
             run_norm(e, L.pre_mixer, h.pre_mixer_norm.kind, X.alpha1, cur, S.normed, rows, d, nullptr);
         } else { // dynamic-tanh norm + token shift
@@ -244,7 +293,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             RUN("dyn_tanh_norm+shift", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
         }
         const uint32_t H = h.num_heads, hd = h.head_dim, vd = h.value_head_dim, rank = h.latent_rank;
-        run_linear(e, lin(S, L.qkv, S.normed, S.q, rows)); // the packed projection of the mixer (queries first)
+        run_linear(e, lin(S, L.qkv, mix_in, S.q, rows)); // the packed projection of the mixer (queries first)
         if (h.mixer_kind == UZU_MIXER_GATED_LRU) {
             const uint32_t w = h.lru_width, bw = w / h.lru_blocks;
             k::GatedLruParams gp{};
@@ -265,8 +314,9 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             const uint32_t G = h.num_groups, ldq = L.qkv.n;
             void* const* vcaches = S.d_cache2_ptrs + (size_t)l * S.max_seqs;
             k::RopeAppendParams rp{};
-            rp.qkv = S.q, rp.ld = ldq, rp.k_col = H * hd, rp.v_col = H * hd + G * hd, rp.heads = H, rp.kv_heads = h.is_kv_sharing ? 0u : G, rp.dim = hd, rp.vdim = vd;
+            rp.qkv = S.q, rp.ld = ldq, rp.k_col = H * hd, rp.v_col = h.values_are_keys ? H * hd : H * hd + G * hd, rp.heads = H, rp.kv_heads = h.is_kv_sharing ? 0u : G, rp.dim = hd, rp.vdim = vd;
             rp.rope_dim = h.use_rope ? L.rope_dim : 0u, rp.cosines = L.rope_cos, rp.sines = L.rope_sin, rp.key_scale = h.key_scale != 0.0f ? h.key_scale : 1.0f;
+            rp.norm_whole = h.qk_norm_whole, rp.interleaved = h.rope_interleaved;
             rp.key_caches = caches, rp.value_caches = vcaches, rp.cache_bf16 = bf, rp.spans = S.d_spans, rp.row_seq = S.d_row_seq, rp.rows = rows;
             rp.q_norm = L.qn.present ? L.qn.scales : nullptr, rp.k_norm = L.kn.present && !h.is_kv_sharing ? L.kn.scales : nullptr, rp.norm_eps = L.qn.present ? L.qn.eps : L.kn.eps;
             RUN("rope_append", (size_t)rows * ldq * 8, k::rope_append(s, rp));
@@ -274,9 +324,12 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             ap.q = S.q, ap.ldq = ldq, ap.out = S.attn, ap.key_caches = caches, ap.value_caches = vcaches, ap.cache_bf16 = bf, ap.sinks = X.sinks, ap.spans = S.d_spans;
             ap.row_seq = S.d_row_seq, ap.rows = rows, ap.heads = H, ap.kv_heads = G, ap.dim = hd, ap.vdim = vd, ap.window = h.sliding_window_size;
             ap.scale = h.attention_scale != 0.0f ? h.attention_scale : 1.0f / sqrtf((float)hd), ap.soft_cap = h.score_soft_cap, ap.nseq = nseq;
+            ap.chunk = h.attention_chunk_size, ap.head_scale = X.head_temp, ap.dist_bias = X.dist_bias, ap.dist_rows = X.dist_rows;
+            if (h.has_gate) ap.gate = S.q + H * hd + (h.is_kv_sharing ? 0u : G * hd + (h.values_are_keys ? 0u : G * vd)), ap.ldgate = ldq; // the gate rows stand behind the values
             for (uint32_t i = 0; i < nseq; ++i) ap.tiles += (counts[i] * (H / G) + 127) / 128;
             // decode-sized passes: spread a tile's key blocks over workgroups (a constant of the layer, so that a captured step stays valid as the context grows)
-            const uint32_t keys = h.sliding_window_size ? h.sliding_window_size : m->d.max_context_length;
+            uint32_t keys = h.sliding_window_size ? h.sliding_window_size : m->d.max_context_length;
+            if (h.attention_chunk_size) keys = std::min(keys, h.attention_chunk_size);
             if (rows <= 4 * S.max_seqs && rows * H <= 4096) ap.splits = std::min<uint32_t>(16, (keys + 31) / 32), ap.split_ws = S.att_ws, ap.split_ws_bytes = S.att_ws_bytes;
             RUN("window_attention", (size_t)rows * H * (hd + vd) * 4, k::window_attention(s, ap));
         } else if (h.mixer_kind == UZU_MIXER_RETENTION) {
@@ -296,7 +349,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         } else {
         // rd: the rotated key part every head shares; the cache row is [latent | rotated part] (kw wide), a query head [plain | rotated] (qw wide)
         const uint32_t rd = h.latent_rope_dim, kw = rank + rd, qw = hd + rd, ldq = L.qkv.n;
-        if (!h.is_kv_sharing && !h.latent_packed) run_linear(e, lin(S, L.lat_down, S.normed, S.ckv, rows));
+        if (!h.is_kv_sharing && !h.latent_packed) run_linear(e, lin(S, L.lat_down, mix_in, S.ckv, rows));
         if (!rd && !h.latent_packed) {
             if (!h.is_kv_sharing)
                 RUN("latent_norm_append", (size_t)rows * rank * 6,
@@ -347,7 +400,41 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             run_linear(e, p);
         }
         } // latent attention
-        if (L.post_mixer.present) { // the mixer's result joins the stream behind its own norm (and the layer scale)
+        if (h.pair_mixer) { // the second mixer beside the first: a delta rule with a decay per head and key channel, reading the same rows
+            const uint32_t Hd = h.dn_num_heads, Gd = h.dn_num_groups, dk = h.dn_head_dim, dv = h.dn_value_head_dim, taps = h.dn_kernel_size, ldi = L.in_proj.n;
+            const uint32_t conv_dim = 2 * Gd * dk + Hd * dv, b_col = conv_dim, a_col = b_col + Hd, g_col = a_col + h.dn_decay_rank;
+            run_linear(e, lin(S, L.in_proj, mix_in, S.dn_in, rows)); // q | k | v | beta | decay down | gate down
+            k::CausalConvParams cp{};
+            cp.x = S.dn_in, cp.ldx = ldi, cp.out = S.dn_cv, cp.ldo = conv_dim, cp.w = L.conv_w, cp.bias = L.conv_b, cp.channels = conv_dim, cp.taps = taps, cp.act = 1;
+            cp.states = S.d_pair_conv_ptrs + (size_t)l * S.max_seqs, cp.spans = S.d_spans, cp.row_seq = S.d_row_seq, cp.nseq = nseq, cp.rows = rows;
+            RUN("causal_conv_rows", (size_t)rows * conv_dim * 4 * (taps + 1), k::causal_conv_rows(s, cp));
+            if (taps > 1) RUN("causal_conv_commit", (size_t)nseq * conv_dim * 8 * (taps - 1), k::causal_conv_commit(s, cp));
+            {   // the low-rank factors' second halves: what enters the recurrence is never rounded, true f32 products in both precisions
+                k::LinearF32Params up = lin(S, X.decay_up, S.dn_in + a_col, S.dn_decay, rows);
+                up.ldx = ldi, up.bf16_products = 0;
+                run_linear(e, up);
+                k::LinearF32Params gu = lin(S, X.gate_up, S.dn_in + g_col, S.dn_gate, rows);
+                gu.ldx = ldi, gu.bf16_products = 0;
+                run_linear(e, gu);
+            }
+            k::ChannelDeltaParams dp{};
+            dp.qkv = S.dn_cv, dp.ld = conv_dim, dp.q_col = 0, dp.k_col = Gd * dk, dp.v_col = 2 * Gd * dk, dp.decay = S.dn_decay, dp.beta = S.dn_in + b_col, dp.ldbeta = ldi;
+            dp.a_log = L.a_log, dp.dt_bias = L.dt_bias, dp.unit_eps = 1e-6f, dp.out = S.dn_o, dp.states = S.d_pair_state_ptrs + (size_t)l * S.max_seqs, dp.spans = S.d_spans;
+            dp.nseq = nseq, dp.rows = rows, dp.heads = Hd, dp.groups = Gd, dp.dim = dk, dp.vdim = dv;
+            RUN("channel_delta_prep", (size_t)rows * (conv_dim + Hd * dk) * 8, k::channel_delta_prep(s, dp));
+            RUN("channel_delta", (size_t)rows * (conv_dim + Hd * (dk + dv)) * 4 + (size_t)nseq * Hd * dk * dv * 8, k::channel_delta(s, dp));
+            k::HeadNormGateParams np{};
+            np.x = S.dn_o, np.ldx = Hd * dv, np.weight = L.dn_norm, np.gate = S.dn_gate, np.ldgate = Hd * dv, np.gate_sigmoid = 1, np.eps = h.dn_norm_epsilon, np.rows = rows, np.heads = Hd, np.width = dv;
+            RUN("head_norm_gate_rows", (size_t)rows * Hd * dv * 12, k::head_norm_gate_rows(s, np));
+            // tmp = scale_main * out(main) + scale_second * out(second)
+            k::LinearF32Params o1 = lin(S, L.out, S.attn, S.tmp, rows);
+            o1.y_scale = h.pair_scale_main;
+            run_linear(e, o1);
+            k::LinearF32Params o2 = lin(S, L.out_proj, S.dn_o, S.tmp, rows);
+            o2.y_scale = h.pair_scale_second, o2.residual = S.tmp, o2.ldr = d;
+            run_linear(e, o2);
+            add_normed(S.tmp, cur, slot, L.post_mixer, X.ls1, nullptr);
+        } else if (L.post_mixer.present) { // the mixer's result joins the stream behind its own norm (and the layer scale)
             run_linear(e, lin(S, L.out, S.attn, S.tmp, rows));
             add_normed(S.tmp, cur, slot, L.post_mixer, X.ls1, pre_mlp_fused ? &L.pre_mlp : (h.no_mlp && !h.has_ple) ? next_pre : nullptr);
             normed_ready = h.no_mlp && !h.has_ple && next_pre;
@@ -358,36 +445,40 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         }
         if (!h.no_mlp) {
             // a parallel block's MLP reads the rows the mixer read (still in S.normed) and adds to the same sum; otherwise the MLP has its own norm of the sum so far
-            if (!h.parallel_block && !pre_mlp_fused) run_norm(e, L.pre_mlp, h.pre_mlp_norm.kind, X.alpha2, slot, S.normed, rows, d, nullptr);
+            const float* mlp_in = h.parallel_block ? mix_in : S.normed;
+            if (!h.parallel_block && !L.pre_mlp.present) mlp_in = conv_input(l, slot, X.in_conv_mlp, h.input_conv_taps, 1); // no pre norm: the stream itself (+ its convolution)
+            else if (!h.parallel_block && !pre_mlp_fused) run_norm(e, L.pre_mlp, h.pre_mlp_norm.kind, X.alpha2, slot, S.normed, rows, d, nullptr);
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
                 const uint32_t E = M.num_routed_experts, top = M.num_active_experts, ff = M.expert_hidden_dim;
                 const k::ExpertAct act = expert_act(M);
                 if (M.routing == UZU_MOE_ROUTE_SCORES) {
                     RUN("moe_route_scores", (size_t)(E + M.num_identity_experts) * d * 2,
-                        k::moe_route_scores(s, S.normed, L.moe.router_weights, X.selection_bias, S.moe_ids, S.moe_w, rows, d, E + M.num_identity_experts, top));
+                        k::moe_route_scores(s, mlp_in, L.moe.router_weights, X.selection_bias, S.moe_ids, S.moe_w, rows, d, E + M.num_identity_experts, top));
                 } else {
-                    RUN("moe_route_topk", (size_t)E * d * 2, k::moe_route_topk(s, S.normed, L.moe.router_weights, L.moe.router_biases, S.moe_ids, S.moe_w, rows, d, E, top, M.router_renorm));
+                    RUN("moe_route_topk", (size_t)E * d * 2, k::moe_route_topk(s, mlp_in, L.moe.router_weights, L.moe.router_biases, S.moe_ids, S.moe_w, rows, d, E, top, M.router_renorm));
                 }
                 k::MoeGroupedParams gp{};
-                gp.x = S.normed, gp.ids = S.moe_ids, gp.weights = S.moe_w, gp.w13 = L.moe.w13, gp.w2 = L.moe.w2, gp.residual = slot, gp.y = slot, gp.y1 = S.moe_y1, gp.hidden = S.hid;
+                gp.x = mlp_in, gp.ids = S.moe_ids, gp.weights = S.moe_w, gp.w13 = L.moe.w13, gp.w2 = L.moe.w2, gp.residual = slot, gp.y = slot, gp.y1 = S.moe_y1, gp.hidden = S.hid;
                 gp.y2 = S.moe_y2, gp.perm = S.moe_perm, gp.slot_pos = S.moe_slot_pos, gp.offsets = S.moe_offsets, gp.cursor = S.moe_cursor;
                 gp.rows = rows, gp.d = d, gp.ff = ff, gp.routed = E, gp.top = top, gp.act = act;
                 if (bf && k::moe_experts_grouped_supported(gp)) { // prefill-sized: buckets per expert through the matrix-core linear
                     RUN("moe_experts_grouped", (size_t)E * 3 * ff * d * 2 + (size_t)rows * top * (3 * ff + 2 * d) * 4, k::moe_experts_grouped(s, gp));
                 } else {
-                    RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, S.normed, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf, act));
+                    RUN("moe_experts_gate_up", (size_t)rows * top * 2 * ff * d * 2, k::moe_experts_gate_up(s, mlp_in, S.moe_ids, L.moe.w13, S.hid, rows, d, ff, E, top, bf, act));
                     RUN("moe_experts_down_combine", (size_t)rows * top * ff * d * 2,
-                        k::moe_experts_down_combine(s, S.hid, S.normed, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
+                        k::moe_experts_down_combine(s, S.hid, mlp_in, S.moe_ids, S.moe_w, L.moe.w2, slot, slot, rows, d, ff, E, top, bf));
                 }
             } else {
                 if (h.mlp_plain) {
-                    k::LinearF32Params up = lin(S, L.up, S.normed, S.hid, rows);
+                    k::LinearF32Params up = lin(S, L.up, mlp_in, S.hid, rows);
                     up.act = 1;
                     run_linear(e, up);
                 } else { // gated: [up ; gate] rows of one projection, then the clamped gate product
-                    run_linear(e, lin(S, L.up, S.normed, S.y1, rows));
-                    RUN("gated_act_rows", (size_t)rows * h.hidden_dim * 12, k::gated_act_rows(s, S.y1, S.hid, rows, h.hidden_dim, expert_act(h.moe)));
+                    run_linear(e, lin(S, L.up, mlp_in, S.y1, rows));
+                    k::ExpertAct ga = expert_act(h.moe);
+                    ga.gelu = h.activation == UZU_ACT_GELU_APPROX ? 1u : 0u;
+                    RUN("gated_act_rows", (size_t)rows * h.hidden_dim * 12, k::gated_act_rows(s, S.y1, S.hid, rows, h.hidden_dim, ga));
                 }
                 if (L.post_mlp.present) {
                     run_linear(e, lin(S, L.down, S.hid, S.tmp, rows));
@@ -423,6 +514,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         run_norm(e, m->output_norm, m->d.output_norm.kind, S.alpha_out, cur, S.out_normed, n_out, d, S.d_out_rows);
         k::LinearF32Params head = lin(S, m->d.tied_embeddings ? m->embedding : m->output_embedding, S.out_normed, S.logits, n_out);
         if (m->d.logit_scale != 1.0f) head.y_scale = m->d.logit_scale; // (0 = a description that never set it)
+        head.soft_cap = m->d.logit_soft_cap;
         run_linear(e, head);
         S.last_logit_rows = n_out;
     }
@@ -501,7 +593,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     auto rms_vec = [](const uzu_norm_desc& n) { return n.present && n.kind == UZU_NORM_STATISTICS && n.scales && !n.subtract_mean && !n.biases; };
     auto norm_ok = [&](const uzu_norm_desc& n) { return n.present && ((n.kind == UZU_NORM_DYNAMIC_TANH && n.scales) || n.kind == UZU_NORM_RMS_SCALAR || rms_vec(n)); };
     UZU_REQUIRE(norm_ok(desc->output_norm), "model_create: an f32-stream design ends in a dynamic-tanh norm or an RMS norm (one gain, or a weight vector)");
-    UZU_UNSUPPORTED(desc->embedding_norm.present || desc->logit_soft_cap != 0.0f, "model_create: decoder options of the bf16-stream families on an f32-stream design");
+    UZU_UNSUPPORTED(desc->embedding_norm.present, "model_create: decoder options of the bf16-stream families on an f32-stream design");
+    auto groups_ok = [&](const uzu_norm_desc& n, uint32_t dim) { return n.groups <= 1 || (rms_vec(n) && dim % n.groups == 0); };
+    UZU_REQUIRE(groups_ok(desc->output_norm, d), "model_create: a norm in parts is an RMS norm with a weight vector over model_dim %% groups == 0 coordinates");
+    if (desc->bigram_buckets)
+        UZU_REQUIRE(desc->bigram_table.weights && desc->bigram_table.method == UZU_QUANT_NONE && desc->bigram_table.n == desc->bigram_buckets + 1 && desc->bigram_table.k == d,
+                    "model_create: the hashed token-pair table is a full-precision matrix [buckets + 1, model_dim]");
     if (desc->has_ple) { // the side table alone: a layer's token input is its slice of the token's row
         UZU_UNSUPPORTED(desc->ple_model_projection.weights || desc->ple_projection_norm.present, "model_create: an f32-stream design's per-layer token input has no model projection");
         UZU_REQUIRE(desc->ple_dim && desc->ple_token_embedding.weights && desc->ple_token_embedding.method == UZU_QUANT_NONE && desc->ple_token_embedding.n == desc->ple_vocab_size &&
@@ -512,8 +609,17 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = desc->layers[l];
         UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION && h.mixer_kind != UZU_MIXER_ATTENTION && h.mixer_kind != UZU_MIXER_RETENTION && h.mixer_kind != UZU_MIXER_GATED_LRU,
-                        "model_create: layer %u: an f32-stream design's mixer is latent attention, attention over cached keys and values, retention, or a gated linear recurrent unit", l);
-        UZU_REQUIRE(norm_ok(h.pre_mixer_norm), "model_create: layer %u needs a dynamic-tanh or RMS pre-mixer norm", l);
+                        "model_create: layer %u: an f32-stream design's mixer is latent attention, attention over cached keys and values, retention, or a gated linear recurrent unit "
+                        "(a channel-decay delta rule rides beside attention as the second mixer of a pair)", l);
+        UZU_UNSUPPORTED(h.mixer_kind != UZU_MIXER_ATTENTION && (h.qk_norm_whole || h.attention_chunk_size || h.values_are_keys || h.rel_bias_rows || h.head_temperature || h.pair_mixer),
+                        "model_create: layer %u: chunks, a distance bias, head temperatures, values that are keys, a whole-projection norm and a second mixer are options of attention", l);
+        UZU_REQUIRE(!h.pre_mixer_norm.present || norm_ok(h.pre_mixer_norm), "model_create: layer %u: a pre-mixer norm is a dynamic-tanh or RMS norm (absent: the mixer reads the stream)", l);
+        UZU_REQUIRE(groups_ok(h.pre_mixer_norm, d) && groups_ok(h.post_mixer_norm, d) && groups_ok(h.pre_mlp_norm, d) && groups_ok(h.post_mlp_norm, d),
+                    "model_create: layer %u: a norm in parts is an RMS norm with a weight vector over model_dim %% groups == 0 coordinates", l);
+        UZU_REQUIRE(!(h.input_conv_mixer || h.input_conv_mlp) || (h.input_conv_taps >= 1 && h.input_conv_taps <= 64), "model_create: layer %u: an input convolution of 1 .. 64 taps", l);
+        UZU_UNSUPPORTED((h.input_conv_mixer && h.pre_mixer_norm.present) || (h.input_conv_mlp && (h.pre_mlp_norm.present || h.parallel_block || h.no_mlp)),
+                        "model_create: layer %u: an input convolution feeds a sublayer that reads the stream itself (no pre norm)", l);
+        UZU_UNSUPPORTED(!h.pre_mixer_norm.present && h.stream_reentry.weights, "model_create: layer %u: a re-entry projection in front of a mixer without a pre norm", l);
         UZU_UNSUPPORTED(h.token_shift && h.pre_mixer_norm.kind != UZU_NORM_DYNAMIC_TANH, "model_create: layer %u: the token shift follows a dynamic-tanh norm", l);
         UZU_REQUIRE(!h.post_mixer_norm.present || rms_vec(h.post_mixer_norm), "model_create: layer %u: a post-mixer norm is an RMS norm with a weight vector", l);
         UZU_REQUIRE(!h.post_mlp_norm.present || (rms_vec(h.post_mlp_norm) && !h.no_mlp && h.mlp_kind != UZU_MLP_MOE && !h.parallel_block),
@@ -554,7 +660,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             UZU_REQUIRE((!desc->num_ropes || h.rope_index < desc->num_ropes) && R.kind != UZU_ROPE_NONE && R.head_dim && R.head_dim % 2 == 0 &&
                         (latent ? R.head_dim == h.latent_rope_dim : R.head_dim <= h.head_dim),
                         "model_create: layer %u: its rotation must turn an even number of at most head_dim coordinates (latent attention: exactly the rotated key part)", l);
-            UZU_UNSUPPORTED(h.rope_interleaved && !latent, "model_create: layer %u: interleaved pairs are the latent attention's rotation", l);
+            UZU_UNSUPPORTED(h.rope_interleaved && !latent && h.mixer_kind != UZU_MIXER_ATTENTION, "model_create: layer %u: interleaved pairs are a rotation of latent attention and attention", l);
         }
         UZU_REQUIRE(h.mixer_kind != UZU_MIXER_LATENT_ATTENTION || (h.latent_rope_dim != 0) == (h.use_rope != 0), "model_create: layer %u: a rotated key part and its rotation come together", l);
         if (h.mixer_kind == UZU_MIXER_LATENT_ATTENTION) {
@@ -578,19 +684,33 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             }
         } else if (h.mixer_kind == UZU_MIXER_ATTENTION) {
             UZU_REQUIRE(h.num_groups && h.num_heads % h.num_groups == 0, "model_create: layer %u: %u query heads on %u key / value heads", l, h.num_heads, h.num_groups);
-            UZU_UNSUPPORTED(h.has_gate, "model_create: layer %u: an output gate is an option of the bf16-stream attention and of latent attention", l);
             UZU_REQUIRE((!h.query_norm.present || h.query_norm.scales) && (!h.key_norm.present || h.key_norm.scales) &&
                         (!h.query_norm.present || !h.key_norm.present || h.query_norm.epsilon == h.key_norm.epsilon),
-                        "model_create: layer %u: query / key norms carry weights [head_dim] and one epsilon", l);
+                        "model_create: layer %u: query / key norms carry weights [head_dim] (or, over the whole projection, [heads head_dim] / [groups head_dim]) and one epsilon", l);
+            UZU_REQUIRE(!h.values_are_keys || (h.value_head_dim == h.head_dim && !h.is_kv_sharing), "model_create: layer %u: values that are the key rows have the keys' width and a cache of their own", l);
+            if (h.rel_bias_rows)
+                UZU_REQUIRE(h.rel_bias && (h.rel_bias_rows == 1 || h.rel_bias_max > (float)(h.rel_bias_rows / 2)), "model_create: layer %u: a distance bias [rows, heads] whose last bucket starts beyond rows / 2", l);
+            if (h.pair_mixer) {
+                const uint32_t Hd = h.dn_num_heads, Gd = h.dn_num_groups, dk = h.dn_head_dim, dv = h.dn_value_head_dim;
+                UZU_UNSUPPORTED(h.pair_mixer != 1 + UZU_MIXER_DELTA_NET || !h.dn_channel_decay, "model_create: layer %u: the second mixer of a pair is a delta rule with channel decays", l);
+                UZU_REQUIRE(h.post_mixer_norm.present && !h.parallel_block, "model_create: layer %u: a pair of mixers joins the stream behind a post-mixer norm", l);
+                UZU_REQUIRE(Hd && Gd && Hd % Gd == 0 && dk && dv && h.dn_kernel_size >= 1 && h.dn_kernel_size <= 64 && h.dn_decay_rank && h.dn_gate_rank,
+                            "model_create: layer %u: the delta rule's %u value heads on %u query / key heads, 1 .. 64 taps, low-rank decay and gate", l, Hd, Gd);
+                UZU_UNSUPPORTED(!k::channel_delta_supported(dk, dv), "model_create: layer %u: delta-rule heads of %u x %u (keys up to 256)", l, dk, dv);
+                UZU_REQUIRE(full(h.dn_in_proj, 2 * Gd * dk + Hd * dv + Hd + h.dn_decay_rank + h.dn_gate_rank, d) && !h.dn_in_proj.out_biases && full(h.dn_out_proj, d, Hd * dv) &&
+                            full(h.dn_decay_up, Hd * dk, h.dn_decay_rank) && full(h.dn_gate_up, Hd * dv, h.dn_gate_rank) && !h.dn_decay_up.out_biases && !h.dn_gate_up.out_biases &&
+                            h.dn_conv_weights && h.dn_a_log && h.dn_dt_bias && h.dn_norm_scales,
+                            "model_create: layer %u: the delta rule's packed projection q | k | v | beta | decay down | gate down, out projection, up factors, convolution, a_log, dt_bias and norm", l);
+            }
             if (h.is_kv_sharing) {
                 UZU_REQUIRE(h.kv_source_layer_index < l, "model_create: layer %u shares the cache of layer %u, which does not precede it", l, h.kv_source_layer_index);
                 const uzu_layer_desc& src = desc->layers[h.kv_source_layer_index];
                 UZU_REQUIRE(src.mixer_kind == UZU_MIXER_ATTENTION && !src.is_kv_sharing && src.num_groups == h.num_groups && src.head_dim == h.head_dim && src.value_head_dim == h.value_head_dim,
                             "model_create: layer %u: the source layer %u must own a cache of the same key / value heads and widths", l, h.kv_source_layer_index);
-                UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim, d), "model_create: layer %u reads another layer's cache: its projection yields queries only", l);
+                UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim + (h.has_gate ? h.num_heads : 0), d), "model_create: layer %u reads another layer's cache: its projection yields queries only (+ gates)", l);
             } else {
-                UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim + h.num_groups * (h.head_dim + h.value_head_dim), d),
-                            "model_create: layer %u: the packed projection must be a full-precision matrix [heads head_dim + groups (head_dim + value_head_dim), model_dim]", l);
+                UZU_REQUIRE(full(h.qkv_projection, h.num_heads * h.head_dim + h.num_groups * (h.head_dim + (h.values_are_keys ? 0 : h.value_head_dim)) + (h.has_gate ? h.num_heads : 0), d),
+                            "model_create: layer %u: the packed projection must be a full-precision matrix [heads head_dim + groups (head_dim + value_head_dim) (+ heads gate rows), model_dim]", l);
             }
         } else if (h.mixer_kind == UZU_MIXER_RETENTION) {
             UZU_REQUIRE(full(h.qkv_projection, 2 * h.num_heads * h.head_dim + 2 * h.num_heads * h.value_head_dim, d) && !h.qkv_projection.out_biases,
@@ -604,7 +724,8 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         UZU_REQUIRE(!(h.has_sinks && h.unit_sink), "model_create: layer %u: sink logits and a unit sink exclude each other", l);
         UZU_REQUIRE(!h.depth_weights || h.num_depth_weights == l + 2, "model_create: layer %u: a depth mix takes %u weights", l, l + 2);
         if (!h.no_mlp) {
-            UZU_REQUIRE(h.parallel_block ? !h.pre_mlp_norm.present : norm_ok(h.pre_mlp_norm), "model_create: layer %u: a pre-MLP norm (dynamic tanh or one-gain RMS), and none in a parallel block", l);
+            UZU_REQUIRE(h.parallel_block ? !h.pre_mlp_norm.present : (!h.pre_mlp_norm.present || norm_ok(h.pre_mlp_norm)),
+                        "model_create: layer %u: a pre-MLP norm is a dynamic-tanh or RMS norm (absent: the MLP reads the stream), and none in a parallel block", l);
             if (h.mlp_kind == UZU_MLP_MOE) {
                 const uzu_moe_desc& M = h.moe;
                 UZU_REQUIRE((M.routing == UZU_MOE_ROUTE_SCORES || M.routing == UZU_MOE_ROUTE_TOPK_LOGITS) && M.num_active_experts &&
@@ -616,8 +737,9 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
                 UZU_REQUIRE(h.activation == UZU_ACT_RELU_SQUARED && full(h.up_projection, h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim),
                             "model_create: layer %u: the plain dense block is down(relu(up x + b)^2) + b with full-precision matrices", l);
             } else {
-                UZU_REQUIRE(h.activation == UZU_ACT_SILU && h.hidden_dim && full(h.up_projection, 2 * h.hidden_dim, d) && full(h.down_projection, d, h.hidden_dim) && !h.parallel_block,
-                            "model_create: layer %u: the gated dense block is down(act(gate) * (up + offset)) with full-precision matrices [up ; gate] and [model_dim, hidden]", l);
+                UZU_REQUIRE((h.activation == UZU_ACT_SILU || h.activation == UZU_ACT_GELU_APPROX) && h.hidden_dim && full(h.up_projection, 2 * h.hidden_dim, d) &&
+                            full(h.down_projection, d, h.hidden_dim) && !h.parallel_block,
+                            "model_create: layer %u: the gated dense block is down(act(gate) * (up + offset)), act = the sigmoid gate or the tanh gelu, with full-precision matrices [up ; gate] and [model_dim, hidden]", l);
             }
         }
     }
@@ -645,6 +767,8 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     m->layers.resize(nl);
     S.layers.resize(nl);
     uint32_t w_q = 0, w_rank = 0, w_lat = 0, w_attn = 0, w_hid = 0, w_top = 1, w_moe = 0, w_routed = 0, w_lru = 0, w_side = 0, w_y1 = 0;
+    uint32_t w_dn_in = 0, w_dn_cv = 0, w_dn_k = 0, w_dn_v = 0;
+    bool any_pair = false, any_inconv = false;
     for (uint32_t l = 0; l < nl; ++l) {
         const uzu_layer_desc& h = desc->layers[l];
         DLayer& L = m->layers[l];
@@ -688,9 +812,45 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             TRY(upload_norm(m, h.ple_norm, d, &L.ple_norm));
         }
         if (h.mixer_kind == UZU_MIXER_ATTENTION) {
-            TRY(upload_norm(m, h.query_norm, h.head_dim, &L.qn));
-            TRY(upload_norm(m, h.key_norm, h.head_dim, &L.kn));
+            TRY(upload_norm(m, h.query_norm, h.qk_norm_whole ? h.num_heads * h.head_dim : h.head_dim, &L.qn));
+            TRY(upload_norm(m, h.key_norm, h.qk_norm_whole ? h.num_groups * h.head_dim : h.head_dim, &L.kn));
+            if (h.head_temperature) TRY(upload(m, h.head_temperature, (size_t)h.num_heads * 4, &X.head_temp));
+            if (h.rel_bias_rows) { // the bias by distance: the bucket rule once, in double, for every distance up to the one the last bucket starts at
+                const uint32_t B = h.rel_bias_rows, E = B / 2, H = h.num_heads;
+                const uint32_t far = B == 1 ? 0u : (uint32_t)ceil((double)h.rel_bias_max);
+                std::vector<float> tab((size_t)(far + 1) * H);
+                for (uint32_t n = 0; n <= far; ++n) {
+                    uint32_t b = n;
+                    if (n >= E) {
+                        b = B - 1;
+                        if (B > 1 && (double)n < (double)h.rel_bias_max) {
+                            const double steps = floor(log((double)n / (double)E) / log((double)h.rel_bias_max / (double)E) * (double)(B - E));
+                            b = std::min<uint32_t>(B - 1, E + (uint32_t)std::max(steps, 0.0));
+                        }
+                    }
+                    for (uint32_t a = 0; a < H; ++a) tab[(size_t)n * H + a] = bf16_to_f32(h.rel_bias[(size_t)b * H + a]);
+                }
+                X.dist_rows = far + 1;
+                TRY(upload(m, tab.data(), tab.size() * 4, &X.dist_bias));
+            }
+            if (h.pair_mixer) {
+                const size_t conv_dim = 2 * (size_t)h.dn_num_groups * h.dn_head_dim + (size_t)h.dn_num_heads * h.dn_value_head_dim;
+                TRY(upload_linear(m, h.dn_in_proj, &L.in_proj));
+                TRY(upload_linear(m, h.dn_out_proj, &L.out_proj));
+                TRY(upload_linear(m, h.dn_decay_up, &X.decay_up));
+                TRY(upload_linear(m, h.dn_gate_up, &X.gate_up));
+                TRY(upload(m, h.dn_conv_weights, conv_dim * h.dn_kernel_size * 4, &L.conv_w));
+                if (h.dn_conv_biases) TRY(upload(m, h.dn_conv_biases, conv_dim * 4, &L.conv_b));
+                TRY(upload(m, h.dn_a_log, (size_t)h.dn_num_heads * 4, &L.a_log));
+                TRY(upload(m, h.dn_dt_bias, (size_t)h.dn_num_heads * h.dn_head_dim * 4, &L.dt_bias));
+                TRY(upload(m, h.dn_norm_scales, (size_t)h.dn_value_head_dim * 4, &L.dn_norm));
+                w_dn_in = std::max(w_dn_in, h.dn_in_proj.n), w_dn_cv = std::max<uint32_t>(w_dn_cv, (uint32_t)conv_dim);
+                w_dn_k = std::max(w_dn_k, h.dn_num_heads * h.dn_head_dim), w_dn_v = std::max(w_dn_v, h.dn_num_heads * h.dn_value_head_dim);
+            }
         }
+        if (h.input_conv_mixer) TRY(upload(m, h.input_conv_mixer, (size_t)d * h.input_conv_taps * 4, &X.in_conv_mixer));
+        if (h.input_conv_mlp) TRY(upload(m, h.input_conv_mlp, (size_t)d * h.input_conv_taps * 4, &X.in_conv_mlp));
+        any_pair |= h.pair_mixer != 0, any_inconv |= h.input_conv_mixer || h.input_conv_mlp;
         if (h.mixer_kind == UZU_MIXER_GATED_LRU) {
             const size_t w = h.lru_width, bw = w / h.lru_blocks;
             TRY(upload(m, h.dn_conv_weights, w * h.dn_kernel_size * 4, &L.conv_w));
@@ -754,6 +914,7 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         }
     }
     if (desc->has_ple) TRY(upload_linear(m, desc->ple_token_embedding, &m->ple_token_embedding, true));
+    if (desc->bigram_buckets) TRY(upload(m, desc->bigram_table.weights, ((size_t)desc->bigram_buckets + 1) * d * 2, &S.pair_table));
     if (!desc->tied_embeddings) TRY(upload_linear(m, desc->output_embedding, &m->output_embedding));
     {   // one table pair per distinct rotation; a layer points at its own
         const uint32_t n_ropes = desc->num_ropes ? desc->num_ropes : (desc->rope.kind != UZU_ROPE_NONE ? 1u : 0u);
@@ -798,6 +959,13 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
         TRY(need_f32(m, R * 2 * w_lru, &S.lru_g));
     }
     if (w_side) TRY(need_f32(m, R * w_side, &S.side_g));
+    if (w_dn_in) {
+        TRY(need_f32(m, R * w_dn_in, &S.dn_in));
+        TRY(need_f32(m, R * w_dn_cv, &S.dn_cv));
+        TRY(need_f32(m, R * w_dn_k, &S.dn_decay));
+        TRY(need_f32(m, R * w_dn_v, &S.dn_gate));
+        TRY(need_f32(m, R * w_dn_v, &S.dn_o));
+    }
     TRY(need_f32(m, R * w_top, &S.moe_w));
     if (w_moe && !S.full_f32) { // workspaces of the grouped expert form (bf16 products only)
         void* q = nullptr;
@@ -816,6 +984,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p)); S.d_cache_ptrs = (void**)p;
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p)); S.d_cache2_ptrs = (void**)p;
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_shift_ptrs = (float**)p;
+    if (any_pair) {
+        TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_pair_state_ptrs = (float**)p;
+        TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_pair_conv_ptrs = (float**)p;
+    }
+    if (any_inconv) { TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_inconv_ptrs = (float**)p; }
+    if (desc->bigram_buckets) { TRY(dev_alloc(m, S.max_seqs * sizeof(uint32_t*), &p)); S.d_prev_tok_ptrs = (uint32_t**)p; }
     TRY(dev_alloc(m, R * 4, &p)); m->batch_tokens = (uint32_t*)p;
     if (flags & UZU_MODEL_DEBUG_TAPS) TRY(need_f32(m, (size_t)nl * R * d, &S.taps));
     {
@@ -887,6 +1061,17 @@ uzu_status s32_state_layer(uzu_hip_model* m, uzu_hip_state* st, uint32_t l) {
     if (h.token_shift) {
         UZU_PROPAGATE(state_alloc(st, (size_t)m->d.model_dim * 4, &p));
         st->layers[l].shift_prev = (float*)p;
+    }
+    if (h.pair_mixer) { // the second mixer's state and convolution window; both read only behind position 0
+        UZU_PROPAGATE(state_alloc(st, (size_t)h.dn_num_heads * h.dn_head_dim * h.dn_value_head_dim * 4, &p, false));
+        st->layers[l].ssm_state = (float*)p;
+        const size_t conv_dim = 2 * (size_t)h.dn_num_groups * h.dn_head_dim + (size_t)h.dn_num_heads * h.dn_value_head_dim;
+        UZU_PROPAGATE(state_alloc(st, conv_dim * (h.dn_kernel_size > 1 ? h.dn_kernel_size - 1 : 1) * 4, &p, false));
+        st->layers[l].conv_state = (float*)p;
+    }
+    if ((h.input_conv_mixer || h.input_conv_mlp) && h.input_conv_taps > 1) { // the mixer's window, then the MLP's; read only behind position 0
+        UZU_PROPAGATE(state_alloc(st, (size_t)2 * (h.input_conv_taps - 1) * m->d.model_dim * 4, &p, false));
+        st->layers[l].in_conv = (float*)p;
     }
     return UZU_OK;
 }

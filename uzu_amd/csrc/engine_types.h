@@ -59,6 +59,7 @@ struct DNorm {
     // PostLayerScalar (encodable_block/normalization.rs:17-21,76-80): 0 None, 1 ScaleResidualSum(scalar), 2 ScaleOutput(scalar)
     int scalar_mode = 0;
     float scalar = 1.0f;
+    uint32_t groups = 1; // f32-stream designs: the row is normed in this many equal consecutive parts
 };
 struct DLayer {
     uzu_layer_desc d; // scalars only (pointers are host pointers: never dereferenced after create)
@@ -126,9 +127,11 @@ struct uzu_hip_state {
         // (bf16 or f32); a retention layer: the f32 state [heads][head_dim][value_head_dim]
         void *cache_k = nullptr, *cache_v = nullptr;
         float* ret_state = nullptr;
+        float* in_conv = nullptr; // the windows of the sublayers' input convolutions: f32 [2][taps - 1][model_dim] (the mixer's, the MLP's)
     };
     std::vector<Layer> layers;
     uint32_t *d_ctx_len = nullptr, *d_tokens = nullptr, *d_out_token = nullptr, *d_sampled = nullptr;
+    uint32_t* prev_token = nullptr; // a model with a hashed token-pair table: the sequence's last token (device)
     uint32_t context_length = 0;
     hipGraphExec_t graph_single = nullptr, graph_two = nullptr;
     uint32_t graph_epoch = 0; // sampling_epoch of the model when the graphs were captured (they bake the sampling kernels in)

@@ -128,6 +128,7 @@ __global__ void __launch_bounds__(256) linear_mfma_kernel(LinearF32Params p) {
                     v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
                 }
                 if (p.y_scale != 0.0f) v *= p.y_scale;
+                if (p.soft_cap != 0.0f) v = p.soft_cap * tanhf(v / p.soft_cap);
                 if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)row * p.ldgate + z]));
                 if (p.mul_table) {
                     uint32_t t = p.mul_tokens[row];

@@ -46,13 +46,43 @@ __global__ void __launch_bounds__(256) embed_rows_f32_kernel(const uint32_t* tok
     for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) dst[i] = bf16_to_f32(src[i]) * scale; // (scale 1: the value itself)
 }
 
+// the same rows plus a hashed (previous token, token) row of a second table; the previous token of a sequence's first row of the pass is the state's
+// (prev[z]), position 0 reads the table's last row
+__global__ void __launch_bounds__(256) embed_pair_rows_f32_kernel(EmbedPairParams p) {
+    const uint32_t r = blockIdx.x;
+    const uint32_t z = p.row_seq[r];
+    const SeqSpan sp = p.spans[z];
+    const uint32_t i = r - sp.row0;
+    uint32_t t = p.tokens[r];
+    if (t >= p.vocab) t = 0;
+    uint32_t row = p.buckets;
+    if (sp.start + i > 0) {
+        uint32_t before = i ? p.tokens[r - 1] : *p.prev[z];
+        if (before >= p.vocab) before = 0;
+        row = (uint32_t)(((uint64_t)before * p.mul_prev + (uint64_t)t * p.mul_cur) % p.buckets);
+    }
+    const uint16_t* src = p.table + (size_t)t * p.d;
+    const uint16_t* add = p.pair_table + (size_t)row * p.d;
+    float* dst = p.out + (size_t)r * p.d;
+    for (uint32_t c = threadIdx.x; c < p.d; c += blockDim.x) dst[c] = bf16_to_f32(src[c]) * p.scale + bf16_to_f32(add[c]);
+}
+// thread = sequence: its last token of the pass becomes the state's previous token (a launch of its own: the rows above read the old one)
+__global__ void __launch_bounds__(64) embed_pair_commit_kernel(EmbedPairParams p, uint32_t nseq) {
+    const uint32_t z = blockIdx.x * 64 + threadIdx.x;
+    if (z >= nseq) return;
+    const SeqSpan sp = p.spans[z];
+    *p.prev[z] = p.tokens[sp.row0 + sp.count - 1];
+}
+
 constexpr int kNormUnroll = 8;
 // a workgroup per row: the sum of squares as 256 strided partial sums folded in a fixed tree, then the scaled row
+// (blockIdx.y = the part of a row that is normed in gridDim.y equal consecutive parts: `d` is the part's width, `ld` the row's)
 __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t d,
-                                                            float offset) {
+                                                            float offset, uint32_t ld) {
     __shared__ float s_red[256];
-    const uint32_t r = blockIdx.x;
-    const float* xr = x + (size_t)(row_index ? row_index[r] : r) * d;
+    const uint32_t r = blockIdx.x, part0 = blockIdx.y * d;
+    const float* xr = x + (size_t)(row_index ? row_index[r] : r) * ld + part0;
+    if (scales) scales += part0;
     float acc = 0.0f;
     for (uint32_t i = threadIdx.x; i < d; i += 256) acc = fmaf(xr[i], xr[i], acc);
     s_red[threadIdx.x] = acc;
@@ -62,7 +92,7 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, floa
         __syncthreads();
     }
     const float inv = 1.0f / sqrtf(s_red[0] / (float)d + eps);
-    float* o = out + (size_t)r * d;
+    float* o = out + (size_t)r * ld + part0;
     // kNormUnroll elements per thread and step, every load of a step in front of its stores (out may alias x for the compiler: a loop of load -> store pairs would
     // pay one memory round trip per element, which is what a one-row decode step's launch consists of)
     for (uint32_t i0 = threadIdx.x; i0 < d; i0 += 256 * kNormUnroll) {
@@ -86,10 +116,12 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* x, floa
 // the same sum of squares over a sublayer's result y; the normed row joins the stream: out = residual + y * inv * (scales + offset) * layer_scale
 // ... and, with `next`, the norm of the new row for the sublayer that follows (its own weights, offset and epsilon): next[r] = rms(out[r]) * (next_scales + next_offset)
 __global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale,
-                                                                float eps, uint32_t d, float* next, const float* next_scales, float next_offset, float next_eps) {
+                                                                float eps, uint32_t d, float* next, const float* next_scales, float next_offset, float next_eps, uint32_t ld) {
     __shared__ float s_red[256];
-    const uint32_t r = blockIdx.x;
-    const float* yr = y + (size_t)r * d;
+    const uint32_t r = blockIdx.x, part0 = blockIdx.y * d; // (a row normed in gridDim.y parts of width d; `next` only with one part)
+    const float* yr = y + (size_t)r * ld + part0;
+    scales += part0;
+    if (layer_scale) layer_scale += part0;
     float acc = 0.0f;
     for (uint32_t i = threadIdx.x; i < d; i += 256) acc = fmaf(yr[i], yr[i], acc);
     s_red[threadIdx.x] = acc;
@@ -99,8 +131,8 @@ __global__ void __launch_bounds__(256) rms_norm_add_rows_kernel(const float* y, 
         __syncthreads();
     }
     const float inv = 1.0f / sqrtf(s_red[0] / (float)d + eps);
-    const float* res = residual + (size_t)r * d;
-    float* o = out + (size_t)r * d;
+    const float* res = residual + (size_t)r * ld + part0;
+    float* o = out + (size_t)r * ld + part0;
     float acc2 = 0.0f;
     for (uint32_t i0 = threadIdx.x; i0 < d; i0 += 256 * kNormUnroll) { // (loads of a step in front of its stores, as in rms_norm_rows_kernel; sums in the same order)
         float yv[kNormUnroll], rv[kNormUnroll], sv[kNormUnroll], lv[kNormUnroll];
@@ -189,6 +221,7 @@ __global__ void __launch_bounds__(256) depth_mix_kernel(const float* slots, size
 
 __device__ __forceinline__ float expert_act(float gate, float up, const ExpertAct& a) {
     const float g = fminf(fmaxf(gate, a.gate_min), a.gate_max), u = fminf(fmaxf(up, a.up_min), a.up_max);
+    if (a.gelu) return gelu_tanh_f32(g) * (u + a.up_offset);
     return g / (1.0f + expf(-(a.alpha * g))) * (u + a.up_offset);
 }
 
@@ -203,6 +236,7 @@ __device__ __forceinline__ float apply_act(float v, uint32_t act) {
 // what follows the activation: the product's scale, a per-(row, product) sigmoid gate
 __device__ __forceinline__ float apply_tail(float v, const LinearF32Params& p, uint32_t r, uint32_t z) {
     if (p.y_scale != 0.0f) v *= p.y_scale;
+    if (p.soft_cap != 0.0f) v = p.soft_cap * tanhf(v / p.soft_cap);
     if (p.gate) v *= 1.0f / (1.0f + expf(-p.gate[(size_t)r * p.ldgate + z]));
     return v;
 }
@@ -550,19 +584,31 @@ uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t*
     return launch_check([&] { hipLaunchKernelGGL(embed_rows_f32_kernel, dim3(rows), dim3(256), 0, s, tokens, table, out, vocab, d, scale); }, "embed_rows_f32");
 }
 
+uzu_status embed_pair_rows_f32(hipStream_t s, const EmbedPairParams& p) {
+    if (!p.rows) return UZU_OK;
+    UZU_REQUIRE(p.tokens && p.table && p.pair_table && p.out && p.spans && p.row_seq && p.prev && p.buckets && p.nseq, "embed_pair_rows_f32: null argument");
+    UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(embed_pair_rows_f32_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "embed_pair_rows_f32"));
+    return launch_check([&] { hipLaunchKernelGGL(embed_pair_commit_kernel, dim3((p.nseq + 63) / 64), dim3(64), 0, s, p, p.nseq); }, "embed_pair_commit");
+}
+
 uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d,
-                         float offset) {
+                         float offset, uint32_t groups) {
     if (!rows) return UZU_OK;
     UZU_REQUIRE(x && out && d, "rms_norm_rows: null argument");
-    return launch_check([&] { hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, s, x, out, scales, gain, eps, row_index, d, offset); }, "rms_norm_rows");
+    if (!groups) groups = 1;
+    UZU_REQUIRE(d % groups == 0 && groups <= 65535, "rms_norm_rows: %u coordinates in %u parts", d, groups);
+    return launch_check([&] { hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows, groups), dim3(256), 0, s, x, out, scales, gain, eps, row_index, d / groups, offset, d); },
+                        "rms_norm_rows");
 }
 
 uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
-                             uint32_t rows, uint32_t d, float* next, const float* next_scales, float next_offset, float next_eps) {
+                             uint32_t rows, uint32_t d, float* next, const float* next_scales, float next_offset, float next_eps, uint32_t groups) {
     if (!rows) return UZU_OK;
     UZU_REQUIRE(y && residual && out && scales && d && (!next || next_scales), "rms_norm_add_rows: null argument");
-    return launch_check([&] { hipLaunchKernelGGL(rms_norm_add_rows_kernel, dim3(rows), dim3(256), 0, s, y, residual, out, scales, offset, layer_scale, eps, d, next, next_scales,
-                                                 next_offset, next_eps); }, "rms_norm_add_rows");
+    if (!groups) groups = 1;
+    UZU_REQUIRE(d % groups == 0 && groups <= 65535 && (groups == 1 || !next), "rms_norm_add_rows: %u coordinates in %u parts (the following norm only behind an undivided one)", d, groups);
+    return launch_check([&] { hipLaunchKernelGGL(rms_norm_add_rows_kernel, dim3(rows, groups), dim3(256), 0, s, y, residual, out, scales, offset, layer_scale, eps, d / groups, next,
+                                                 next_scales, next_offset, next_eps, d); }, "rms_norm_add_rows");
 }
 
 uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act) {

@@ -28,7 +28,34 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeAppendParams p) {
     const uint32_t half = p.rope_dim / 2;
     const float* cs = p.cosines + (size_t)t * p.rope_dim;
     const float* sn = p.sines + (size_t)t * p.rope_dim;
-    if (p.q_norm || p.k_norm) { // a wave per head: x <- x / sqrt(mean(x^2) + eps) * w over the head's coordinates, in front of the rotation
+    // values first, as projected: with v_col == k_col the values are the keys in front of their norm and rotation
+    if (p.kv_heads && p.value_caches) {
+        void* vc = p.value_caches[z];
+        const size_t vrow = (size_t)t * p.kv_heads * p.vdim;
+        for (uint32_t idx = threadIdx.x; idx < p.kv_heads * p.vdim; idx += 256) cache_st(vc, p.cache_bf16, vrow + idx, row[p.v_col + idx]);
+        __syncthreads();
+    }
+    if (p.norm_whole && (p.q_norm || p.k_norm)) { // one RMS norm over all query coordinates of the row, one over all key coordinates: 256 strided partial sums, a fixed tree
+        __shared__ float s_red[256];
+        for (int pass = 0; pass < 2; ++pass) {
+            const float* w = pass ? p.k_norm : p.q_norm;
+            const uint32_t n = pass ? p.kv_heads * p.dim : p.heads * p.dim;
+            if (!w || !n) continue;
+            float* h = pass ? row + p.k_col : row;
+            float ss = 0.0f;
+            for (uint32_t i = threadIdx.x; i < n; i += 256) ss = fmaf(h[i], h[i], ss);
+            s_red[threadIdx.x] = ss;
+            __syncthreads();
+            for (uint32_t wd = 128; wd > 0; wd >>= 1) {
+                if (threadIdx.x < wd) s_red[threadIdx.x] += s_red[threadIdx.x + wd];
+                __syncthreads();
+            }
+            const float inv = 1.0f / sqrtf(s_red[0] / (float)n + p.norm_eps);
+            __syncthreads();
+            for (uint32_t i = threadIdx.x; i < n; i += 256) h[i] = h[i] * inv * w[i];
+        }
+        __syncthreads();
+    } else if (p.q_norm || p.k_norm) { // a wave per head: x <- x / sqrt(mean(x^2) + eps) * w over the head's coordinates, in front of the rotation
         const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         for (uint32_t a = wave; a < p.heads + p.kv_heads; a += 4) {
             const bool is_q = a < p.heads;
@@ -46,9 +73,10 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeAppendParams p) {
     for (uint32_t idx = threadIdx.x; idx < p.heads * half; idx += 256) {
         const uint32_t a = idx / half, i = idx - a * half;
         float* h = row + (size_t)a * p.dim;
-        const float u = h[i], v = h[i + half], c = cs[i], s = sn[i];
-        h[i] = u * c - v * s;
-        h[i + half] = v * c + u * s;
+        const uint32_t iu = p.interleaved ? 2 * i : i, iv = p.interleaved ? 2 * i + 1 : i + half;
+        const float u = h[iu], v = h[iv], c = cs[i], s = sn[i];
+        h[iu] = u * c - v * s;
+        h[iv] = v * c + u * s;
     }
     if (!p.kv_heads) return;
     const float ks = p.key_scale;
@@ -57,21 +85,17 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeAppendParams p) {
     for (uint32_t idx = threadIdx.x; idx < p.kv_heads * p.dim; idx += 256) {
         const uint32_t g = idx / p.dim, c = idx - g * p.dim;
         float* h = row + p.k_col + (size_t)g * p.dim;
-        if (c < half) {
-            const float u = h[c], v = h[c + half], co = cs[c], s = sn[c];
-            const float a = (u * co - v * s) * ks, b = (v * co + u * s) * ks;
-            if (kc) cache_st(kc, p.cache_bf16, krow + idx, a), cache_st(kc, p.cache_bf16, krow + idx + half, b);
-            else h[c] = a, h[c + half] = b;
-        } else if (c >= p.rope_dim) {
+        if (c >= p.rope_dim) {
             const float a = h[c] * ks;
             if (kc) cache_st(kc, p.cache_bf16, krow + idx, a);
             else h[c] = a;
+        } else if (p.interleaved ? (c & 1) == 0 : c < half) { // the thread of a pair's first coordinate turns the pair
+            const uint32_t step = p.interleaved ? 1 : half, i = p.interleaved ? c >> 1 : c;
+            const float u = h[c], v = h[c + step], co = cs[i], s = sn[i];
+            const float a = (u * co - v * s) * ks, b = (v * co + u * s) * ks;
+            if (kc) cache_st(kc, p.cache_bf16, krow + idx, a), cache_st(kc, p.cache_bf16, krow + idx + step, b);
+            else h[c] = a, h[c + step] = b;
         }
-    }
-    if (p.value_caches) {
-        void* vc = p.value_caches[z];
-        const size_t vrow = (size_t)t * p.kv_heads * p.vdim;
-        for (uint32_t idx = threadIdx.x; idx < p.kv_heads * p.vdim; idx += 256) cache_st(vc, p.cache_bf16, vrow + idx, row[p.v_col + idx]);
     }
 }
 
@@ -89,7 +113,9 @@ __global__ void __launch_bounds__(64) window_attention_simple_kernel(WindowAtten
     const uint32_t g = a / (p.heads / p.kv_heads);
     const void* K = p.key_caches[z];
     const void* V = p.value_caches[z];
-    const uint32_t lo = (p.window && t + 1 > p.window) ? t + 1 - p.window : 0u;
+    uint32_t lo = (p.window && t + 1 > p.window) ? t + 1 - p.window : 0u;
+    if (p.chunk) lo = max(lo, t / p.chunk * p.chunk);
+    const float hscale = p.head_scale ? p.scale * p.head_scale[a] : p.scale;
     const float* q = p.q + (size_t)r * p.ldq + (size_t)a * p.dim;
     for (uint32_t c = lane; c < p.dim; c += 64) s_q[c] = q[c];
     __syncthreads();
@@ -123,8 +149,9 @@ __global__ void __launch_bounds__(64) window_attention_simple_kernel(WindowAtten
                 const float* kr = (const float*)K + base;
                 for (uint32_t c = 0; c < p.dim; ++c) dot = fmaf(s_q[c], kr[c], dot);
             }
-            s = dot * p.scale;
+            s = dot * hscale;
             if (p.soft_cap != 0.0f) s = p.soft_cap * tanhf(s / p.soft_cap);
+            if (p.dist_bias) s += p.dist_bias[(size_t)min(t - j, p.dist_rows - 1) * p.heads + a];
         }
         const float m_new = fmaxf(m, wave_max(s));
         const float w = j <= t ? expf(s - m_new) : 0.0f;
@@ -146,11 +173,12 @@ __global__ void __launch_bounds__(64) window_attention_simple_kernel(WindowAtten
         }
     }
     float* o = p.out + ((size_t)r * p.heads + a) * p.vdim;
+    const float og = p.gate ? 1.0f / (1.0f + expf(-p.gate[(size_t)r * p.ldgate + a])) : 1.0f;
 #pragma unroll
     for (uint32_t i = 0; i < kMaxVecPerLane; ++i) {
         const uint32_t c = lane + 64 * i;
         if (c >= p.vdim) break;
-        o[c] = acc[i] / l;
+        o[c] = p.gate ? acc[i] / l * og : acc[i] / l;
     }
 }
 
@@ -161,6 +189,7 @@ uzu_status rope_append(hipStream_t s, const RopeAppendParams& p) {
     UZU_REQUIRE(p.qkv && p.spans && p.row_seq && p.heads && p.dim, "rope_append: null argument");
     UZU_REQUIRE(p.rope_dim % 2 == 0 && p.rope_dim <= p.dim && (!p.rope_dim || (p.cosines && p.sines)), "rope_append: rotation width %u of a head of %u (even, with its tables)", p.rope_dim, p.dim);
     UZU_REQUIRE(!p.kv_heads || ((p.key_caches != nullptr) == (p.value_caches != nullptr)), "rope_append: key and value caches come together");
+    UZU_REQUIRE(p.v_col != p.k_col || !p.kv_heads || (p.vdim == p.dim && p.value_caches), "rope_append: values that are the key rows have the keys' width and go to a cache");
     return launch_check([&] { hipLaunchKernelGGL(rope_append_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "rope_append");
 }
 
@@ -171,6 +200,7 @@ uzu_status window_attention(hipStream_t s, const WindowAttentionParams& p) {
     UZU_REQUIRE(p.q && p.out && p.key_caches && p.value_caches && p.spans && p.row_seq, "window_attention: null argument");
     UZU_REQUIRE(p.heads && p.kv_heads && p.heads % p.kv_heads == 0 && p.dim && p.vdim, "window_attention: %u query heads on %u key / value heads", p.heads, p.kv_heads);
     UZU_UNSUPPORTED(p.vdim > 64 * kMaxVecPerLane || p.dim > 8192, "window_attention: value width %u (at most %u)", p.vdim, 64 * kMaxVecPerLane);
+    UZU_REQUIRE(!p.dist_bias || p.dist_rows, "window_attention: a distance bias without its rows");
     if (p.form == 2 || (p.form == 0 && window_attention_mfma_supported(p))) {
         UZU_UNSUPPORTED(!window_attention_mfma_supported(p), "window_attention: the matrix-core form does not take this shape");
         return window_attention_mfma(s, p);

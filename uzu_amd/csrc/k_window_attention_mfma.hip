@@ -45,7 +45,11 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
     }
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const uint32_t items = sp.count * hg;
-    auto row_lo = [&](uint32_t t) { return (p.window && t + 1 > p.window) ? t + 1 - p.window : 0u; };
+    auto row_lo = [&](uint32_t t) { // the first key the row at position t sees: the window's edge or its chunk's start, whichever is later
+        uint32_t lo = (p.window && t + 1 > p.window) ? t + 1 - p.window : 0u;
+        if (p.chunk) lo = max(lo, t / p.chunk * p.chunk);
+        return lo;
+    };
     // this lane's item
     const uint32_t it = wg * 128 + wave * 32 + l32;
     const bool valid = it < items;
@@ -88,6 +92,7 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
     const uint8_t* vc = (const uint8_t*)p.value_caches[z];
     const size_t kpitch = (size_t)p.kv_heads * p.dim, vpitch = (size_t)p.kv_heads * p.vdim;
     const float inv_cap = p.soft_cap != 0.0f ? 1.0f / p.soft_cap : 0.0f;
+    const float hscale = p.head_scale ? p.scale * p.head_scale[head] : p.scale;
 
     const uint32_t kstep = SPLIT ? 32 * gridDim.z : 32;
     for (uint32_t kb = kmin + (SPLIT ? 32 * blockIdx.z : 0); kb <= kmax; kb += kstep) {
@@ -123,11 +128,12 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
         for (int r = 0; r < 16; ++r) {
             const uint32_t key = kb + (r & 3) + 8 * (r >> 2) + 4 * half;
             const bool ok = valid && key >= lo && key <= t;
-            float sc = st[r] * p.scale;
+            float sc = st[r] * hscale;
             if (p.soft_cap != 0.0f) { // cap * tanh(s / cap), tanh(x) = 1 - 2 / (1 + e^(2x))
                 const float e2 = fast_exp(2.0f * sc * inv_cap);
                 sc = p.soft_cap * (1.0f - 2.0f / (1.0f + e2));
             }
+            if (p.dist_bias && ok) sc += p.dist_bias[(size_t)min(t - key, p.dist_rows - 1) * p.heads + head];
             st[r] = ok ? sc : -INFINITY;
             mx = fmaxf(mx, st[r]);
         }
@@ -174,7 +180,8 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
         if (half == 0) ws[RP] = m_run, ws[RP + 1] = l_run;
         return;
     }
-    const float inv = 1.0f / l_run;
+    float inv = 1.0f / l_run;
+    if (p.gate) inv *= 1.0f / (1.0f + expf(-p.gate[(size_t)(sp.row0 + row) * p.ldgate + head]));
     float* out = p.out + ((size_t)(sp.row0 + row) * p.heads + head) * p.vdim;
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -186,13 +193,16 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(WindowAttent
 }
 
 // a workgroup per item: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the splits, in split order (a split that saw no key has l = 0 and m = -1e30)
-__global__ void __launch_bounds__(128) window_attention_merge_kernel(const float* ws, float* out, uint32_t splits, uint32_t vdim, uint32_t rp) {
+// (gate: the item's result times sigmoid(gate[row, head]), item = row * heads + head)
+__global__ void __launch_bounds__(128) window_attention_merge_kernel(const float* ws, float* out, uint32_t splits, uint32_t vdim, uint32_t rp, const float* gate, uint32_t ldgate,
+                                                                     uint32_t heads) {
     const uint32_t item = blockIdx.x, tid = threadIdx.x;
     const float* base = ws + (size_t)item * splits * (rp + 4);
     float M = -1.0e30f;
     for (uint32_t s = 0; s < splits; ++s) M = fmaxf(M, base[(size_t)s * (rp + 4) + rp]);
     float den = 0.0f;
     for (uint32_t s = 0; s < splits; ++s) den = fmaf(fast_exp(base[(size_t)s * (rp + 4) + rp] - M), base[(size_t)s * (rp + 4) + rp + 1], den);
+    if (gate) den *= 1.0f + expf(-gate[(size_t)(item / heads) * ldgate + item % heads]);
     for (uint32_t c = tid; c < vdim; c += 128) {
         float acc = 0.0f;
         for (uint32_t s = 0; s < splits; ++s) acc = fmaf(fast_exp(base[(size_t)s * (rp + 4) + rp] - M), base[(size_t)s * (rp + 4) + c], acc);
@@ -232,7 +242,7 @@ uzu_status window_attention_mfma(hipStream_t s, const WindowAttentionParams& p) 
         else if (nb == 2) UZU_WA(2);
         else UZU_WA(4);
 #undef UZU_WA
-        return launch_check([&] { hipLaunchKernelGGL(window_attention_merge_kernel, dim3(p.rows * p.heads), dim3(128), 0, s, (const float*)p.split_ws, p.out, p.splits, p.vdim, 32 * nb); },
+        return launch_check([&] { hipLaunchKernelGGL(window_attention_merge_kernel, dim3(p.rows * p.heads), dim3(128), 0, s, (const float*)p.split_ws, p.out, p.splits, p.vdim, 32 * nb, p.gate, p.ldgate, p.heads); },
                             "window_attention_merge");
     }
     const dim3 grid(p.tiles, p.kv_heads);

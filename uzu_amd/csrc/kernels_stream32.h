@@ -7,6 +7,8 @@
 //   k_window_attention.hip   rotation + key / value cache append, attention over cached keys and values (grouped heads, score cap, window, sinks)
 //   k_retention.hip          retention: the decayed outer-product state (token by token and in chunks), per-head RMS division + gate
 //   k_gated_lru.hip          the gated linear recurrent unit: short causal convolution over a carried window, gates / decays / state update
+//   k_causal_conv.hip        a causal per-channel convolution of row blocks over a carried window (sublayer inputs, the delta rule's q / k / v), per-head norm + gate
+//   k_channel_delta.hip      the gated delta rule with a decay per head and key channel
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -28,14 +30,34 @@ uzu_status embed_rows_f32(hipStream_t s, const uint32_t* tokens, const uint16_t*
 // RMS norm with one gain: out[r, :] = gain * x[src(r), :] / sqrt(mean(x[src(r), :]^2) + eps),   src(r) = row_index ? row_index[r] : r.
 // scales (f32 [d], optional) multiplies per coordinate on top, as (scales[i] + offset): a weight stored around zero has offset 1.  The row's sum of squares is
 // taken in a fixed order.
+// groups > 1: the row is cut into that many equal consecutive parts and each part is divided by its own root mean square.
 uzu_status rms_norm_rows(hipStream_t s, const float* x, float* out, const float* scales, float gain, float eps, const uint32_t* row_index, uint32_t rows, uint32_t d,
-                         float offset = 0.0f);
+                         float offset = 0.0f, uint32_t groups = 1);
+
+// out[r, :] = f32(table[token[r], :]) * scale + f32(pair_table[pair(r), :]): a second table indexed by a hash of (previous token, token),
+//   pair(r) = (before * mul_prev + token * mul_cur) mod buckets, before = the token in front of r in its sequence -- of this pass, or (at the pass's first row)
+//   the sequence's state *prev[z]; a sequence's position 0 reads row `buckets` (pair_table bf16 [buckets + 1, d]).  A second launch leaves every sequence's
+//   last token of the pass in *prev[z].
+struct EmbedPairParams {
+    const uint32_t* tokens;
+    const uint16_t *table, *pair_table;
+    float* out;
+    uint32_t rows, vocab, d;
+    float scale;
+    uint32_t buckets, mul_prev, mul_cur;
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t* const* prev; // device array [nseq] of device pointers
+    uint32_t nseq;
+};
+uzu_status embed_pair_rows_f32(hipStream_t s, const EmbedPairParams& p);
 
 // A sublayer's result joins the stream behind its own norm:  out[r, :] = residual[r, :] + y[r, :] / sqrt(mean(y[r, :]^2) + eps) * (scales + offset) * layer_scale
 // (scales f32 [d]; layer_scale f32 [d] or null; out may alias residual).  The same fixed-order sum of squares as rms_norm_rows.  With `next` the launch also leaves
 // the norm of the new row for the sublayer that follows: next[r, :] = out[r, :] / sqrt(mean(out[r, :]^2) + next_eps) * (next_scales + next_offset).
 uzu_status rms_norm_add_rows(hipStream_t s, const float* y, const float* residual, float* out, const float* scales, float offset, const float* layer_scale, float eps,
-                             uint32_t rows, uint32_t d, float* next = nullptr, const float* next_scales = nullptr, float next_offset = 0.0f, float next_eps = 0.0f);
+                             uint32_t rows, uint32_t d, float* next = nullptr, const float* next_scales = nullptr, float next_offset = 0.0f, float next_eps = 0.0f,
+                             uint32_t groups = 1); // groups > 1: y is normed in that many equal consecutive parts (no `next` then)
 
 // Dynamic-tanh norm, optionally followed by the token shift:
 //   h[r]   = tanh(alpha * x[src(r)]) * scales + biases          src(r) = row_index ? row_index[r] : r
@@ -76,6 +98,7 @@ struct LinearF32Params {
     uint32_t act;
     uint32_t bf16_products;
     float y_scale;     // != 0: the product (behind bias and act, before the residual) is multiplied by it
+    float soft_cap;    // != 0: ... and then capped, cap * tanh(v / cap) (the read-out's logit cap)
     const float* gate; // batched products: product z of row r is multiplied by sigmoid(gate[r * ldgate + z]) (a scalar gate per head); null = none
     uint32_t ldgate;
     // a multiplier per (row's token, column) behind all of that: y[r, n] *= f32(mul_table[token[r] * mul_ld + mul_col0 + n])  (bf16 table, an id >= mul_vocab reads
@@ -105,8 +128,10 @@ uzu_status moe_route_topk(hipStream_t s, const float* x, const uint16_t* router,
                           uint32_t outputs, uint32_t top, uint32_t renorm);
 // The gated product of an expert's hidden unit: g = clamp(gate, gate_min, gate_max), u = clamp(up, up_min, up_max), g * sigmoid(alpha * g) * (u + up_offset).
 // The default is silu(gate) * up.
+// gelu != 0: the gate's activation is the tanh form of gelu instead of g * sigmoid(alpha * g).
 struct ExpertAct {
     float alpha = 1.0f, gate_min = -INFINITY, gate_max = INFINITY, up_min = -INFINITY, up_max = INFINITY, up_offset = 0.0f;
+    uint32_t gelu = 0;
 };
 // The gated product of a dense block: hidden[r, f] = act(gate = y1[r, ff + f], up = y1[r, f])   (y1 f32 [rows][2 ff]: up rows first, as the packed projection yields them)
 uzu_status gated_act_rows(hipStream_t s, const float* y1, float* hidden, uint32_t rows, uint32_t ff, const ExpertAct& act);
@@ -203,6 +228,7 @@ uzu_status latent_rope_append(hipStream_t s, const LatentRopeAppendParams& p);
 // [positions][kv_heads * dim] and [positions][kv_heads * vdim], bf16 or f32) rotated keys and values go to row t of the sequence's caches; without (null) the
 // keys are replaced in place and values stay where they are.  kv_heads == 0: the row carries queries only (a layer that reads another layer's cache).
 // q_norm / k_norm (f32 [dim], optional): every query / key head is RMS-normed over its dim coordinates (norm_eps, plain weights) in front of the rotation.
+// Values go to the cache first, as the projection left them: v_col == k_col (vdim == dim) makes the values the keys in front of their norm and rotation.
 struct RopeAppendParams {
     float* qkv;
     uint32_t ld, k_col, v_col;
@@ -211,6 +237,8 @@ struct RopeAppendParams {
     float key_scale;
     const float *q_norm, *k_norm;
     float norm_eps;
+    uint32_t norm_whole;  // q_norm / k_norm are f32 [heads * dim] / [kv_heads * dim]: ONE RMS norm over all of a row's query (key) coordinates instead of one per head
+    uint32_t interleaved; // the rotation pairs coordinates (2i, 2i + 1) instead of (i, i + rope_dim / 2)
     void* const* key_caches;
     void* const* value_caches;
     uint32_t cache_bf16;
@@ -236,6 +264,15 @@ struct WindowAttentionParams {
     const uint32_t* row_seq;
     uint32_t rows, heads, kv_heads, dim, vdim, window;
     float scale, soft_cap;
+    // chunk != 0: the row at position t sees keys j <= t of its own chunk only, j >= floor(t / chunk) * chunk (chunks counted from position 0 of the sequence).
+    // head_scale (f32 [heads] or null): the scaled score of head a is multiplied by head_scale[a].  dist_bias (f32 [dist_rows][heads] or null): dist_bias[min(t - j,
+    // dist_rows - 1), a] is added behind scale, head_scale and cap.  gate (f32 rows of pitch ldgate or null): out[r, a, :] is multiplied by sigmoid(gate[r, a]).
+    uint32_t chunk;
+    const float* head_scale;
+    const float* dist_bias;
+    uint32_t dist_rows;
+    const float* gate;
+    uint32_t ldgate;
     uint32_t form;  // 0: chosen by shape; 1: the simple form (a wave per row and head); 2: the matrix-core form
     uint32_t nseq;  // entries of `spans`
     uint32_t tiles; // sum over the sequences of ceil(count * (heads / kv_heads) / 128): the matrix-core form's item tiles (the caller knows the counts)
@@ -310,6 +347,66 @@ struct GatedLruParams {
 size_t lru_piece_ws_bytes(uint32_t pieces, uint32_t width);
 uzu_status lru_conv(hipStream_t s, const GatedLruParams& p);
 uzu_status lru_scan(hipStream_t s, const GatedLruParams& p);
+
+// A causal convolution over positions on every channel of a block of rows (k_causal_conv.hip).  Row r (sequence z, position t), channel c:
+//   out[r, o_col + c] = act(bias[c] + sum_j w[c, j] * xin(t - (taps - 1) + j, c))  (+ x[r, x_col + c] with add_input: a sublayer that reads h + conv(h))
+// xin = channel c of the sequence's input rows `x` (f32, pitch ldx, column x_col): of this pass, or (in front of the pass) the taps - 1 inputs the state keeps
+// (states[z] + state_offset: f32 [taps - 1][channels], oldest first), or zero in front of position 0.  w f32 [channels][taps]: the last tap weighs the row itself.
+// act: 0 none, 1 silu.  `out` is another block of rows than `x`.  causal_conv_commit leaves the last taps - 1 inputs behind the pass in the state; it reads the
+// same `x`, which must still hold the pass's inputs.
+struct CausalConvParams {
+    const float* x;
+    uint32_t ldx, x_col;
+    float* out;
+    uint32_t ldo, o_col;
+    const float *w, *bias;
+    uint32_t channels, taps, add_input, act;
+    float* const* states; // device array [nseq]
+    size_t state_offset;  // floats
+    const SeqSpan* spans;
+    const uint32_t* row_seq;
+    uint32_t nseq, rows;
+};
+uzu_status causal_conv_rows(hipStream_t s, const CausalConvParams& p);
+uzu_status causal_conv_commit(hipStream_t s, const CausalConvParams& p);
+
+// Per head, in place: x[r, a, :] <- x[r, a, :] / sqrt(mean(x[r, a, :]^2) + eps) * weight[:] * gate(g[r, a, :])    (x f32 rows of pitch ldx, heads * width used;
+// weight f32 [width] or null; g f32 rows of pitch ldgate or null; gate = sigmoid (gate_sigmoid) or silu)
+struct HeadNormGateParams {
+    float* x;
+    uint32_t ldx;
+    const float* weight;
+    const float* gate;
+    uint32_t ldgate, gate_sigmoid;
+    float eps;
+    uint32_t rows, heads, width;
+};
+uzu_status head_norm_gate_rows(hipStream_t s, const HeadNormGateParams& p);
+
+// The gated delta rule with a decay per head and key channel (k_channel_delta.hip).  Row r (sequence z) of `qkv` (f32, pitch ld) holds queries [groups][dim] at
+// q_col, keys [groups][dim] at k_col and values [heads][vdim] at v_col (behind their convolution and silu); value head a reads group a / (heads / groups).
+//   channel_delta_prep (in place):  q <- q / sqrt(sum q^2 + unit_eps) * dim^(-1/2),  k <- k / sqrt(sum k^2 + unit_eps)  per head;
+//                                   beta[r, a] <- sigmoid(beta[r, a]);   decay[r, a, c] <- exp(-exp(a_log[a]) * softplus(decay[r, a, c] + dt_bias[a, c]))
+//   channel_delta:                  per head, row after row:  S <- decay * S (rows = key channels),  u = beta (v - S^T k),  S <- S + k u^T,  out[r, a, :] = S^T q
+// states: device array [nseq] of pointers to f32 [heads][dim][vdim], read at the pass's first row (zeros instead when the span starts at position 0) and left
+// behind its last.  decay f32 [rows][heads * dim], beta f32 rows of pitch ldbeta, out f32 [rows][heads * vdim].  All f32; every sum runs in the same order
+// whatever else the pass carries and however the rows were cut into passes.
+struct ChannelDeltaParams {
+    float* qkv;
+    uint32_t ld, q_col, k_col, v_col;
+    float* decay;
+    float* beta;
+    uint32_t ldbeta;
+    const float *a_log, *dt_bias;
+    float unit_eps;
+    float* out;
+    float* const* states;
+    const SeqSpan* spans;
+    uint32_t nseq, rows, heads, groups, dim, vdim;
+};
+bool channel_delta_supported(uint32_t dim, uint32_t vdim);
+uzu_status channel_delta_prep(hipStream_t s, const ChannelDeltaParams& p);
+uzu_status channel_delta(hipStream_t s, const ChannelDeltaParams& p);
 
 } // namespace k
 } // namespace uzu

@@ -40,7 +40,7 @@ class NormDesc(C.Structure):
         ("present", C.c_uint32), ("full_layer", C.c_uint32), ("subtract_mean", C.c_uint32), ("kind", C.c_uint32),
         ("epsilon", C.c_float), ("scale_offset", C.c_float),
         ("scales", C.c_void_p), ("biases", C.c_void_p),
-        ("alpha", C.c_float), ("reserved", C.c_uint32),
+        ("alpha", C.c_float), ("groups", C.c_uint32),
     ]
 
 
@@ -104,6 +104,11 @@ class LayerDesc(C.Structure):
         ("lru_gate_weights", C.c_void_p), ("lru_gate_biases", C.c_void_p), ("lru_lambda", C.c_void_p),
         ("layer_scale_mixer", C.c_void_p), ("layer_scale_mlp", C.c_void_p),
         ("ple_slice", C.c_uint32), ("weights_of_layer", C.c_uint32), ("stream_reentry", LinearDesc),
+        ("input_conv_taps", C.c_uint32), ("qk_norm_whole", C.c_uint32), ("input_conv_mixer", C.c_void_p), ("input_conv_mlp", C.c_void_p),
+        ("attention_chunk_size", C.c_uint32), ("values_are_keys", C.c_uint32), ("rel_bias_rows", C.c_uint32), ("rel_bias_max", C.c_float),
+        ("rel_bias", C.c_void_p), ("head_temperature", C.c_void_p),
+        ("pair_mixer", C.c_uint32), ("pair_scale_main", C.c_float), ("pair_scale_second", C.c_float),
+        ("dn_channel_decay", C.c_uint32), ("dn_decay_rank", C.c_uint32), ("dn_gate_rank", C.c_uint32), ("dn_decay_up", LinearDesc), ("dn_gate_up", LinearDesc),
     ]
 
 
@@ -123,7 +128,7 @@ class ModelDesc(C.Structure):
         ("ple_dim", C.c_uint32), ("ple_vocab_size", C.c_uint32), ("ple_embed_scale", C.c_float),
         ("ple_model_projection_scale", C.c_float), ("ple_input_scale", C.c_float), ("reserved", C.c_uint32),
         ("ple_token_embedding", LinearDesc), ("ple_model_projection", LinearDesc), ("ple_projection_norm", NormDesc),
-        ("f32_stream", C.c_uint32), ("reserved5", C.c_uint32),
+        ("f32_stream", C.c_uint32), ("bigram_buckets", C.c_uint32), ("bigram_mul_prev", C.c_uint32), ("bigram_mul_cur", C.c_uint32), ("bigram_table", LinearDesc),
     ]
 
 
@@ -186,10 +191,11 @@ class NormWeights:
     biases: Optional[np.ndarray] = None
     kind: int = NORM_STATISTICS          # NORM_DYNAMIC_TANH: tanh(alpha * x) * scales + biases; NORM_RMS_SCALAR: alpha * x / sqrt(mean(x^2) + epsilon) (f32-stream designs)
     alpha: float = 0.0
+    groups: int = 0                      # f32-stream designs: the row is normed in this many equal consecutive parts (0 / 1: as a whole)
 
     def desc(self) -> NormDesc:
         return NormDesc(int(self.present), int(self.full_layer), int(self.subtract_mean), int(self.kind), self.epsilon,
-                        self.scale_offset, _ptr(self.scales), _ptr(self.biases), float(self.alpha), 0)
+                        self.scale_offset, _ptr(self.scales), _ptr(self.biases), float(self.alpha), int(self.groups))
 
 
 ABSENT_NORM = NormWeights(present=False)
@@ -341,6 +347,24 @@ class LayerWeights:
     ple_slice: int = 0                             # which ple_dim-wide slice of the side table's row this layer run reads
     weights_of_layer: Optional[int] = None         # this run uses the tensors of that earlier run (a looped stack); its state is its own
     stream_reentry: Optional[LinearWeights] = None  # x <- W [x ; x0] in front of this run, [model_dim, 2 model_dim]
+    # f32-stream designs: sublayers that read h + conv(h) (a causal per-channel convolution of their input rows; pre norms may then be absent)
+    input_conv_taps: int = 0
+    input_conv_mixer: Optional[np.ndarray] = None  # f32 [model_dim, taps]
+    input_conv_mlp: Optional[np.ndarray] = None
+    # attention options: one RMS norm over the whole query / key projection, causal chunks, values = the key rows as projected, a bias per (distance bucket, head),
+    # a temperature per head; has_gate = a sigmoid gate per head from rows behind the packed projection
+    qk_norm_whole: bool = False
+    attention_chunk_size: int = 0
+    values_are_keys: bool = False
+    rel_bias: Optional[np.ndarray] = None          # bf16 bits [rows, heads]
+    rel_bias_max: float = 0.0
+    head_temperature: Optional[np.ndarray] = None  # f32 [heads]
+    # a second mixer beside the first (MIXER_DELTA_NET with a decay per head and key channel: the dn_* fields), result = pair_scales[0] * main + pair_scales[1] * second
+    pair_mixer: Optional[int] = None
+    pair_scales: tuple = (1.0, 1.0)
+    dn_channel_decay: bool = False
+    dn_decay_up: Optional[LinearWeights] = None    # [heads dk, rank]
+    dn_gate_up: Optional[LinearWeights] = None     # [heads dv, rank]
 
     def _moe_desc(self) -> MoeDesc:
         if self.moe is not None:
@@ -380,11 +404,17 @@ class LayerWeights:
             int(self.latent_rope_dim), int(self.latent_packed), int(self.rope_interleaved), int(self.lru_width), int(self.lru_blocks), float(self.lru_decay_rate),
             _ptr(self.lru_gate_weights), _ptr(self.lru_gate_biases), _ptr(self.lru_lambda), _ptr(self.layer_scale_mixer), _ptr(self.layer_scale_mlp),
             int(self.ple_slice), 0 if self.weights_of_layer is None else int(self.weights_of_layer) + 1, ld(self.stream_reentry),
+            int(self.input_conv_taps), int(self.qk_norm_whole), _ptr(self.input_conv_mixer), _ptr(self.input_conv_mlp),
+            int(self.attention_chunk_size), int(self.values_are_keys), 0 if self.rel_bias is None else int(self.rel_bias.shape[0]), float(self.rel_bias_max),
+            _ptr(self.rel_bias), _ptr(self.head_temperature),
+            0 if self.pair_mixer is None else int(self.pair_mixer) + 1, float(self.pair_scales[0]), float(self.pair_scales[1]),
+            int(self.dn_channel_decay), 0 if self.dn_decay_up is None else int(self.dn_decay_up.k), 0 if self.dn_gate_up is None else int(self.dn_gate_up.k),
+            ld(self.dn_decay_up), ld(self.dn_gate_up),
         )
 
     def linears(self):
         names = ("qkv_projection", "gate_projection", "out_projection", "dn_in_proj", "dn_out_proj", "up_projection",
-                 "down_projection", "latent_down", "latent_up_keys", "latent_up_values", "stream_reentry")
+                 "down_projection", "latent_down", "latent_up_keys", "latent_up_values", "stream_reentry", "dn_decay_up", "dn_gate_up")
         out = [(n, getattr(self, n)) for n in names if getattr(self, n) is not None]
         if self.ple is not None:
             out += [("ple.gate", self.ple.gate), ("ple.projection", self.ple.projection)]
@@ -547,6 +577,8 @@ class ModelBundle:
     architecture: Optional[str] = None           # config.json `architecture` of a design that is not in the reference's config schema
     side_table: Optional[LinearWeights] = None   # f32-stream designs: a second token table [vocab, slices * side_dim]; a layer with `ple` reads its slice of the token's row
     side_dim: int = 0
+    bigram: Optional[LinearWeights] = None       # f32-stream designs: a hashed (previous token, token) table [buckets + 1, model_dim] added to the embedding rows
+    bigram_mul: tuple = (0, 0)                   # (multiplier of the previous token, of the token)
     _keep: list = field(default_factory=list, repr=False)
 
     def desc(self) -> ModelDesc:
@@ -563,7 +595,7 @@ class ModelBundle:
             return ModelDesc(self.vocab_size, self.model_dim, len(self.layers), int(self.tied_embeddings), self.input_scale, self.logit_scale, self.logit_soft_cap,
                              self.max_context_length, self.rope.desc(), self.embedding.desc(), out_emb, self.output_norm.desc(), C.cast(arr, C.POINTER(LayerDesc)),
                              len(self.ropes) if self.ropes else 0, 1, C.cast(ropes, C.POINTER(RopeDesc)) if ropes is not None else None, self.embedding_norm.desc(),
-                             int(self.side_dim), int(self.side_table.n), 1.0, 0.0, 0.0, 0, self.side_table.desc(), e, ABSENT_NORM.desc(), int(self.f32_stream), 0)
+                             int(self.side_dim), int(self.side_table.n), 1.0, 0.0, 0.0, 0, self.side_table.desc(), e, ABSENT_NORM.desc(), int(self.f32_stream), *self._bigram_desc())
         return ModelDesc(self.vocab_size, self.model_dim, len(self.layers), int(self.tied_embeddings),
                          self.input_scale, self.logit_scale, self.logit_soft_cap, self.max_context_length,
                          self.rope.desc(), self.embedding.desc(), out_emb, self.output_norm.desc(),
@@ -574,7 +606,12 @@ class ModelBundle:
                          p.ple_dim if p else 0, p.ple_vocab_size if p else 0, p.ple_embed_scale if p else 0.0,
                          p.model_projection_scale if p else 0.0, p.input_scale if p else 0.0, 0,
                          p.token_embedding.desc() if p else e, p.model_projection.desc() if p else e,
-                         (p.projection_norm if p else ABSENT_NORM).desc(), int(self.f32_stream), 0)
+                         (p.projection_norm if p else ABSENT_NORM).desc(), int(self.f32_stream), *self._bigram_desc())
+
+    def _bigram_desc(self):
+        if self.bigram is None:
+            return 0, 0, 0, LinearDesc()
+        return int(self.bigram.n) - 1, int(self.bigram_mul[0]), int(self.bigram_mul[1]), self.bigram.desc()
 
     # ---- algorithmic bytes per decoded token (SURVEY.md §8d formula) ----
     def weight_stream_bytes(self) -> int:

@@ -80,6 +80,8 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
     exact = rows // 2
     if n < exact:
         return n
+    if rows == 1:  # one row for every distance
+        return 0
     return min(rows - 1, exact + int(math.floor(math.log(n / exact) / math.log(far / exact) * (rows - exact))))
 
 
@@ -220,3 +222,132 @@ def forward(cfg: dict, w: Dict[str, np.ndarray], tokens) -> Tuple[np.ndarray, Li
     if cap:
         logits = cap * np.tanh(logits / cap)
     return logits, streams
+
+
+# ------------------------------------------------------------------------------------------------ the tests' own configurations, weights and model directories
+def dense(ff):
+    return {"kind": "dense", "ff": int(ff)}
+
+
+def attention_layer(heads, kv_heads, dim, vdim, rot_dims=0, rot_base=10000.0, scale=None, mlp=None):
+    mx = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": float(scale if scale is not None else dim ** -0.5)}
+    if rot_dims:
+        mx["rot"] = {"dims": int(rot_dims), "base": float(rot_base)}
+    return {"type": "attention", "mixer": mx, "mlp": mlp}
+
+
+def parallel_layer(heads, kv_heads, dim, chunk, rel_rows, bias_max, d_heads, d_kv_heads, d_dim, d_vdim, conv, rank=3, scale=None, left_scale=1.0, right_scale=1.0, mlp=None):
+    """`rel_rows` and `rank` size tensors only (a reader takes them from the shapes): they are kept under '_sizes', which a reader ignores"""
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "mask": {"size": int(chunk)}, "bias_max": float(bias_max),
+            "scale": float(scale if scale is not None else dim ** -0.5)}
+    right = {"heads": d_heads, "kv_heads": d_kv_heads, "dim": d_dim, "vdim": d_vdim, "conv": int(conv)}
+    return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": float(left_scale), "right_scale": float(right_scale)}, "mlp": mlp,
+            "_sizes": {"rel_rows": int(rel_rows), "rank": int(rank)}}
+
+
+def config(vocab, width, layers, eps=1e-5, groups=1, taps=4, embed_scale=1.0, bigram=None, logit_softcap=0.0):
+    """bigram = (buckets, mul_prev, mul_cur)"""
+    em = {"scale": float(embed_scale)}
+    if bigram:
+        em["bigram"] = {"buckets": int(bigram[0]), "mul_prev": int(bigram[1]), "mul_cur": int(bigram[2])}
+    return {"architecture": "Zovolorn", "vocab": int(vocab), "width": int(width), "norm": {"eps": float(eps), "groups": int(groups)}, "canon": {"taps": int(taps)},
+            "embedding": em, "layers": layers, "logit_softcap": float(logit_softcap)}
+
+
+def bf16_bits(a):
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def to_bf16(a):
+    return (bf16_bits(a).astype(np.uint32) << 16).view(np.float32).reshape(np.shape(a))
+
+
+def weights(cfg, seed):
+    """random tensors (bf16-representable f32) for a configuration: products ~ N(0, gain^2 / in), norm weights around 1, decays from fast to slow"""
+    rng = np.random.default_rng(seed)
+    vocab, width, taps = cfg["vocab"], cfg["width"], cfg["canon"]["taps"]
+    W = {}
+
+    def lin(name, n, k, gain=1.0, bias=False):
+        W[name] = to_bf16(rng.standard_normal((n, k)) * gain / np.sqrt(k))
+        if bias:
+            W[name + ".b"] = to_bf16(rng.standard_normal(n) * 0.2)
+
+    def vec(name, n, centre, spread):
+        W[name] = to_bf16(centre + spread * (rng.random(n) - 0.5))
+
+    W["embed"] = to_bf16(rng.standard_normal((vocab, width)) / cfg["embedding"]["scale"])
+    bg = cfg["embedding"].get("bigram")
+    if bg:
+        W["bigram"] = to_bf16(rng.standard_normal((bg["buckets"] + 1, width)) * 0.5)
+    for i, lc in enumerate(cfg["layers"]):
+        p, mx = f"l{i}.", lc["mixer"]
+        vec(p + "norm1", width, 1.0, 0.6)
+        W[p + "canon1"] = to_bf16(rng.standard_normal((width, taps)) * 0.3)
+        if lc["type"] == "attention":
+            H, G, dk, dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+            q = p + "mix."
+            lin(q + "q", H * dk, width, 2.0), lin(q + "k", G * dk, width, 2.0), lin(q + "v", G * dv, width), lin(q + "g", H, width, 2.0)
+            vec(q + "q.norm", H * dk, 1.5, 0.6), vec(q + "k.norm", G * dk, 1.5, 0.6), vec(q + "sink", H, 0.5, 3.0)
+            lin(q + "o", width, H * dv)
+        else:
+            lm, rm, sz = mx["left"], mx["right"], lc["_sizes"]
+            H, G, dk = lm["heads"], lm["kv_heads"], lm["dim"]
+            q = p + "mix.left."
+            lin(q + "q", H * dk, width, 2.0), lin(q + "k", G * dk, width, 2.0)
+            vec(q + "q.norm", dk, 1.5, 0.6), vec(q + "k.norm", dk, 1.5, 0.6), vec(q + "temp", H, 1.0, 1.0)
+            W[q + "rel"] = to_bf16(rng.standard_normal((sz["rel_rows"], H)) * 1.5)
+            lin(q + "o", width, H * dk)
+            Hd, Gd, dk, dv, ct, rank = rm["heads"], rm["kv_heads"], rm["dim"], rm["vdim"], rm["conv"], sz["rank"]
+            q = p + "mix.right."
+            lin(q + "q", Gd * dk, width, 2.0), lin(q + "k", Gd * dk, width, 2.0), lin(q + "v", Hd * dv, width, 1.5), lin(q + "b", Hd, width, 2.0)
+            for n, ch in (("q", Gd * dk), ("k", Gd * dk), ("v", Hd * dv)):
+                W[q + n + ".conv"] = to_bf16(rng.standard_normal((ch, ct)) * 0.6)
+            lin(q + "a1", rank, width), lin(q + "a2", Hd * dk, rank, 2.0), lin(q + "g1", rank, width), lin(q + "g2", Hd * dv, rank, 2.0)
+            vec(q + "A_log", Hd, -1.0, 3.0), vec(q + "dt_bias", Hd * dk, -1.0, 3.0), vec(q + "norm", dv, 1.0, 0.6)
+            lin(q + "o", width, Hd * dv)
+        if lc.get("mlp") is not None:
+            ff = lc["mlp"]["ff"]
+            vec(p + "norm2", width, 1.0, 0.6)
+            W[p + "canon2"] = to_bf16(rng.standard_normal((width, taps)) * 0.3)
+            lin(p + "mlp.gate", ff, width, 1.5, True), lin(p + "mlp.up", ff, width, 1.5, True), lin(p + "mlp.down", width, ff, 1.0, True)
+    vec("final.norm", width, 1.0, 0.6)
+    return W
+
+
+def write_model_dir(path, cfg, W):
+    """config.json + model.safetensors (bf16) in the design's layout, written with nothing but the file format"""
+    import json
+    import os
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(cfg, f)
+    header, blobs, off = {}, [], 0
+    for name in sorted(W):
+        b = bf16_bits(W[name]).tobytes()
+        header[name] = {"dtype": "BF16", "shape": list(np.shape(W[name])), "data_offsets": [off, off + len(b)]}
+        blobs.append(b)
+        off += len(b)
+    hj = json.dumps(header).encode()
+    hj += b" " * (-len(hj) % 8)
+    with open(os.path.join(path, "model.safetensors"), "wb") as f:
+        f.write(len(hj).to_bytes(8, "little") + hj + b"".join(blobs))
+
+
+def logit_error(got, want):
+    """per row: RMS over the vocabulary of the difference with its mean taken off, relative to the RMS of the centred expected row"""
+    d = np.asarray(got, dtype=np.float64) - np.asarray(want, dtype=np.float64)
+    d = d - d.mean(-1, keepdims=True)
+    w = np.asarray(want, dtype=np.float64)
+    w = w - w.mean(-1, keepdims=True)
+    return np.sqrt((d * d).mean(-1)) / np.sqrt((w * w).mean(-1) + 1e-30)
+
+
+def greedy(cfg, W, prompt, n):
+    """n tokens by arg-max, every step a forward pass over the whole sequence"""
+    toks = list(prompt)
+    for _ in range(n):
+        logits, _ = forward(cfg, W, toks)
+        toks.append(int(np.argmax(logits[-1])))
+    return toks[len(prompt):]

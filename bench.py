@@ -12,7 +12,7 @@ Prints ONE JSON line on rank 0 (contract in the task statement) with two extra o
   roofline     -- the dominant kernel (the int4 GEMV family) : algorithmic bytes / HIP-event time, vs 8 TB/s HBM
   cpu_baseline -- the CPU oracle (port of the reference's single-threaded CPU backend) timed on this host
 
-Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix | relulix | begasun (prefill / chained decode / batched
+Side runs (their own JSON line, never the headline): --config c3|c4|c5, --exact, and --design lazolix | relulix | begasun | zovolorn (prefill / chained decode / batched
 decode of an f32-stream design at real layer sizes beside the engine's closest existing model at equal sizes).
 """
 import argparse
@@ -59,11 +59,12 @@ def parse_args():
                     help="BASELINE.json configs[1..4]: c2 (default, the headline) Qwen3.5-0.8B int4 ctx-2048 decode; c3 Llama-3-8B int4, 4k prefill x 8 "
                          "sequences in batched passes (prefill tokens/s, MFMA roofline); c4 Llama-3-8B int8 decode (TP = --gpus); c5 Qwen3-14B-class int4 at "
                          "ctx 8192, one sequence decoding while another is prefilled (TP = --gpus)")
-    ap.add_argument("--design", choices=["", "lazolix", "relulix", "begasun"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
+    ap.add_argument("--design", choices=["", "lazolix", "relulix", "begasun", "zovolorn"], default="", help="side runs of a design outside BASELINE.json (never the headline): `lazolix` times prefill, "
                     "chained decode and batched decode of the f32-stream design at layer sizes of real models (random weights), beside the closest "
                     "bf16-stream model of the engine at equal sizes (windowed attention with sinks + int4 dense / bf16 expert MLPs); `relulix` does the same for the "
                     "design of parallel blocks with rotated attention, retention layers and clamped experts, beside Lazolix with experts at equal sizes; `begasun` for the looped stack of recurrent units, latent attention with a rotated key part "
-                    "and grouped attention, beside Lazolix with dense blocks at equal sizes")
+                    "and grouped attention, beside Lazolix with dense blocks at equal sizes; `zovolorn` for the pairs of chunked attention + channel-decay delta rule alternating with grouped attention, "
+                    "beside Begasun's recurrent units alternating with grouped attention at equal sizes")
     ap.add_argument("--design-sizes", default="w1024,w2048", help="--design: comma-separated size presets")
     ap.add_argument("--sequences", type=int, default=8, help="c3: sequences per batched prefill pass")
     ap.add_argument("--prompt", type=int, default=4096, help="c3: prompt tokens per sequence")
@@ -637,8 +638,48 @@ def bench_begasun(args):
     print(json.dumps(out), flush=True)
 
 
+def bench_zovolorn(args):
+    """Prefill / decode throughput of Zovolorn models (pairs of chunked attention + channel-decay delta rule alternating with grouped attention layers; input
+    convolutions, norms in parts, gelu-gated dense blocks with biases, the hashed token-pair table) beside the closest existing model at equal size: Begasun without
+    its loop and token input, recurrent units alternating with grouped attention (same width / heads / head widths / key-value heads / dense width / vocabulary /
+    layer count; a norm behind every sublayer, a gated dense block, a short convolution in front of the recurrence).  One JSON line."""
+    import tempfile
+    from uzu_amd import begasun, loader, synthetic as S, zovolorn
+    from uzu_amd.backend import Context
+    ctx = Context.new(0)
+    prompt_len, steps, warm, nbatch = 2048, max(8, min(args.steps, 128)), max(2, min(args.warmup, 8)), 8
+    out = {"metric": "zovolorn_side_run", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 products, f32 stream", "data": "synthetic (random weights, synthetic token ids)",
+           "prompt_tokens": prompt_len, "decode_steps": steps, "batched_decode_sequences": nbatch, "sizes": {}}
+    for size in [s for s in args.design_sizes.split(",") if s]:
+        z = LAZOLIX_SIZES[size]
+        prompt = S.synthetic_prompt(prompt_len, z["vocab"]).astype(np.uint32)
+        context = prompt_len + steps + warm + 64
+        H, G, dim, vd = z["heads"], max(1, z["heads"] // 4), z["dim"], z["vdim"]
+        mlp = zovolorn.dense_mlp(z["ff"])
+        par = lambda: zovolorn.parallel_layer(H // 2, G, dim, 256, 32, 1024.0, H // 2, G, dim, vd, 4, rank=64, left_scale=0.6, right_scale=0.9, mlp=mlp)
+        att = lambda: zovolorn.attention_layer(H, G, dim, vd, rot_dims=dim // 2, rot_base=500000.0, mlp=mlp)
+        layers = ([par(), att()] * ((z["layers"] + 1) // 2))[:z["layers"]]
+        cfg = zovolorn.config(z["vocab"], z["width"], layers, groups=4, taps=4, embed_scale=0.5, bigram=(65521, 31, 17), logit_softcap=30.0)
+        with tempfile.TemporaryDirectory() as tmp:
+            zovolorn.save(tmp, cfg, zovolorn.random_tensors(cfg, seed=1))
+            bundle = loader.load_model_dir(tmp, max_context_length=context)
+        bmlp = begasun.dense_mlp(z["ff"], limit=7.0)
+        blayers = ([begasun.rglru_layer(z["width"], H, 4, mlp=bmlp), begasun.attention_layer(H, G, dim, vd, begasun.rotation(dim // 2, 500000.0), mlp=bmlp)] * ((z["layers"] + 1) // 2))[:z["layers"]]
+        bcfg = begasun.config(z["vocab"], z["width"], blayers)
+        with tempfile.TemporaryDirectory() as tmp:
+            begasun.save(tmp, bcfg, begasun.random_tensors(bcfg, seed=1))
+            closest = loader.load_model_dir(tmp, max_context_length=context)
+        rec = {"zovolorn": _time_f32_stream(ctx, bundle, prompt, steps, warm, nbatch), "closest": _time_f32_stream(ctx, closest, prompt, steps, warm, nbatch)}
+        out["sizes"][size] = {"shape": dict(z, kv_heads=G, chunk=256, pair_heads=H // 2, delta_heads=H // 2, delta_kv_heads=G, conv=4, low_rank=64, norm_groups=4, taps=4,
+                                            pattern="(chunked attention + delta rule), grouped attention, ...", closest="recurrent unit, grouped attention, ..."), **rec}
+    ctx.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
+    if args.design == "zovolorn":
+        return bench_zovolorn(args)
     if args.design == "begasun":
         return bench_begasun(args)
     if args.design == "lazolix":

@@ -427,12 +427,19 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             np.x = S.dn_o, np.ldx = Hd * dv, np.weight = L.dn_norm, np.gate = S.dn_gate, np.ldgate = Hd * dv, np.gate_sigmoid = 1, np.eps = h.dn_norm_epsilon, np.rows = rows, np.heads = Hd, np.width = dv;
             RUN("head_norm_gate_rows", (size_t)rows * Hd * dv * 12, k::head_norm_gate_rows(s, np));
             // tmp = scale_main * out(main) + scale_second * out(second)
-            k::LinearF32Params o1 = lin(S, L.out, S.attn, S.tmp, rows);
-            o1.y_scale = h.pair_scale_main;
-            run_linear(e, o1);
-            k::LinearF32Params o2 = lin(S, L.out_proj, S.dn_o, S.tmp, rows);
-            o2.y_scale = h.pair_scale_second, o2.residual = S.tmp, o2.ldr = d;
-            run_linear(e, o2);
+            // (a scale of exactly zero takes its mixer's product out; both zero: a product that vanishes)
+            const bool main_on = h.pair_scale_main != 0.0f, second_on = h.pair_scale_second != 0.0f;
+            if (main_on || !second_on) {
+                k::LinearF32Params o1 = lin(S, L.out, S.attn, S.tmp, rows);
+                o1.y_scale = main_on ? h.pair_scale_main : 1.0e-37f;
+                run_linear(e, o1);
+            }
+            if (second_on) {
+                k::LinearF32Params o2 = lin(S, L.out_proj, S.dn_o, S.tmp, rows);
+                o2.y_scale = h.pair_scale_second;
+                if (main_on) o2.residual = S.tmp, o2.ldr = d;
+                run_linear(e, o2);
+            }
             add_normed(S.tmp, cur, slot, L.post_mixer, X.ls1, nullptr);
         } else if (L.post_mixer.present) { // the mixer's result joins the stream behind its own norm (and the layer scale)
             run_linear(e, lin(S, L.out, S.attn, S.tmp, rows));

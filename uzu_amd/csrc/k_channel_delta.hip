@@ -2,10 +2,10 @@
 //
 // Per value head a (reading query / key group a / (heads / groups)), with S [dk][dv] the head's state:
 //     S <- diag(decay_t) S,   u = beta_t (v_t - S^T k_t),   S <- S + k_t u^T,   o_t = S^T q_t
-// Everything is f32.  The value columns of S never meet: column j only needs k_t, q_t, decay_t, beta_t and v_t[j].  So a workgroup owns 64 columns of one
-// (sequence, head) and four threads share a column, each holding a quarter of its rows in registers; the two dot products of a token are sums over the thread's
-// own rows in row order, then a fixed exchange between the four threads.  The order of every sum is the same whatever else the pass carries and however a prompt
-// was cut: prompts, portions and decode steps run this one kernel.  q, k and decay of a few tokens are staged in LDS for all columns at once.
+// Everything is f32.  The value columns of S never meet: column j only needs k_t, q_t, decay_t, beta_t and v_t[j].  So a workgroup owns 16 columns of one
+// (sequence, head) and sixteen threads share a column, each holding a sixteenth of its rows in registers; the two dot products of a token are sums over the
+// thread's own rows in row order, then a fixed exchange between the sixteen threads.  The order of every sum is the same whatever else the pass carries and however a prompt
+// was cut: prompts, portions and decode steps run this one kernel.  q, k, decay, v and beta of sixteen tokens are staged in LDS for all columns at once.
 #include "device_utils.h"
 #include "kernels_stream32.h"
 
@@ -36,64 +36,94 @@ __global__ void __launch_bounds__(256) channel_delta_prep_kernel(ChannelDeltaPar
     for (uint32_t i = threadIdx.x; i < p.heads; i += 256) b[i] = 1.0f / (1.0f + expf(-b[i]));
 }
 
-constexpr uint32_t kStage = 8; // tokens whose q / k / decay are staged at once
+constexpr int kStage = 16; // tokens whose q / k / decay / v / beta are staged at once
 
-// grid (sequence * heads, ceil(dv / 64)); thread = (column, quarter of the rows); RP = rows per thread (dk <= 4 RP)
+// grid (sequence * heads, ceil(dv / 16)); thread = (column, sixteenth of the rows): a wave owns 4 columns, a workgroup 16.  RP = rows per thread (dk <= 16 RP);
+// thread `part` of a column owns rows part, part + 16, ...  The next stage's rows travel from memory into registers while the current stage is worked on.
 template <int RP>
 __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaParams p) {
-    __shared__ __attribute__((aligned(16))) float s_k[kStage][4 * RP], s_q[kStage][4 * RP], s_g[kStage][4 * RP];
+    constexpr int DK = 16 * RP;
+    __shared__ float s_k[kStage][DK], s_q[kStage][DK], s_g[kStage][DK], s_v[kStage][16], s_b[kStage];
     const uint32_t z = blockIdx.x / p.heads, a = blockIdx.x % p.heads, g = a / (p.heads / p.groups);
-    const uint32_t tid = threadIdx.x, col = blockIdx.y * 64 + (tid >> 2), part = tid & 3;
+    const uint32_t tid = threadIdx.x, cl = tid >> 4, part = tid & 15, col = blockIdx.y * 16 + cl;
     const bool live = col < p.vdim;
     const SeqSpan sp = p.spans[z];
     float* state = p.states[z] + (size_t)a * p.dim * p.vdim;
     float S[RP];
 #pragma unroll
     for (int n = 0; n < RP; ++n) {
-        const uint32_t i = part * RP + n;
+        const uint32_t i = part + 16 * n;
         S[n] = (sp.start && live && i < p.dim) ? state[(size_t)i * p.vdim + col] : 0.0f;
     }
-    for (uint32_t i0 = 0; i0 < sp.count; i0 += kStage) {
-        const uint32_t nt = sp.count - i0 < kStage ? sp.count - i0 : kStage;
-        __syncthreads(); // the stage before has been read
-        for (uint32_t e = tid; e < nt * 4 * RP; e += 256) {
-            const uint32_t tk = e / (4 * RP), i = e - tk * (4 * RP);
+    float pf[3 * RP], pf_v = 0.0f, pf_b = 0.0f;
+    // element e * 256 + tid of a stage's [k | q | decay][token][row] block: rows beyond dk and tokens beyond the share are zeros (zero keys and queries leave the
+    // padding rows of S at zero)
+    auto fetch = [&](uint32_t i0) {
+        const uint32_t nt = sp.count - i0 < (uint32_t)kStage ? sp.count - i0 : (uint32_t)kStage;
+#pragma unroll
+        for (int e = 0; e < 3 * RP; ++e) {
+            const uint32_t rem = (uint32_t)(e % RP) * 256 + tid, tk = rem / DK, i = rem % DK;
             const size_t r = sp.row0 + i0 + tk;
-            const bool in = i < p.dim; // rows beyond dk: zero keys and queries leave the padding rows of S at zero
-            s_k[tk][i] = in ? p.qkv[r * p.ld + p.k_col + (size_t)g * p.dim + i] : 0.0f;
-            s_q[tk][i] = in ? p.qkv[r * p.ld + p.q_col + (size_t)g * p.dim + i] : 0.0f;
-            s_g[tk][i] = in ? p.decay[(r * p.heads + a) * p.dim + i] : 0.0f;
+            float v = 0.0f;
+            if (tk < nt && i < p.dim) {
+                if (e / RP == 0) v = p.qkv[r * p.ld + p.k_col + (size_t)g * p.dim + i];
+                else if (e / RP == 1) v = p.qkv[r * p.ld + p.q_col + (size_t)g * p.dim + i];
+                else v = p.decay[(r * p.heads + a) * p.dim + i];
+            }
+            pf[e] = v;
         }
+        const uint32_t tk = tid >> 4, c = blockIdx.y * 16 + (tid & 15);
+        pf_v = (tk < nt && c < p.vdim) ? p.qkv[(size_t)(sp.row0 + i0 + tk) * p.ld + p.v_col + (size_t)a * p.vdim + c] : 0.0f;
+        pf_b = (tid < nt) ? p.beta[(size_t)(sp.row0 + i0 + tid) * p.ldbeta + a] : 0.0f;
+    };
+    auto put = [&]() {
+#pragma unroll
+        for (int e = 0; e < 3 * RP; ++e) {
+            const uint32_t rem = (uint32_t)(e % RP) * 256 + tid, tk = rem / DK, i = rem % DK;
+            float* dst = e / RP == 0 ? &s_k[0][0] : e / RP == 1 ? &s_q[0][0] : &s_g[0][0];
+            dst[tk * DK + i] = pf[e];
+        }
+        s_v[tid >> 4][tid & 15] = pf_v;
+        if (tid < (uint32_t)kStage) s_b[tid] = pf_b;
+    };
+    fetch(0);
+    for (uint32_t i0 = 0; i0 < sp.count; i0 += kStage) {
+        const uint32_t nt = sp.count - i0 < (uint32_t)kStage ? sp.count - i0 : (uint32_t)kStage;
+        __syncthreads(); // the stage before has been read
+        put();
         __syncthreads();
+        if (i0 + kStage < sp.count) fetch(i0 + kStage);
         for (uint32_t tk = 0; tk < nt; ++tk) {
-            const size_t r = sp.row0 + i0 + tk;
-            const float v = live ? p.qkv[r * p.ld + p.v_col + (size_t)a * p.vdim + col] : 0.0f;
-            const float beta = p.beta[r * p.ldbeta + a];
-            const float *kk = &s_k[tk][part * RP], *qq = &s_q[tk][part * RP], *gg = &s_g[tk][part * RP];
+            const float v = s_v[tk][cl], beta = s_b[tk];
+            const float *kk = &s_k[tk][part], *qq = &s_q[tk][part], *gg = &s_g[tk][part];
             float dot = 0.0f;
 #pragma unroll
             for (int n = 0; n < RP; ++n) {
-                S[n] *= gg[n];
-                dot = fmaf(S[n], kk[n], dot);
+                S[n] *= gg[16 * n];
+                dot = fmaf(S[n], kk[16 * n], dot);
             }
             dot += __shfl_xor(dot, 1, 64);
             dot += __shfl_xor(dot, 2, 64);
+            dot += __shfl_xor(dot, 4, 64);
+            dot += __shfl_xor(dot, 8, 64);
             const float u = beta * (v - dot);
             float o = 0.0f;
 #pragma unroll
             for (int n = 0; n < RP; ++n) {
-                S[n] = fmaf(kk[n], u, S[n]);
-                o = fmaf(S[n], qq[n], o);
+                S[n] = fmaf(kk[16 * n], u, S[n]);
+                o = fmaf(S[n], qq[16 * n], o);
             }
             o += __shfl_xor(o, 1, 64);
             o += __shfl_xor(o, 2, 64);
-            if (live && part == 0) p.out[(r * p.heads + a) * p.vdim + col] = o;
+            o += __shfl_xor(o, 4, 64);
+            o += __shfl_xor(o, 8, 64);
+            if (live && part == 0) p.out[((size_t)(sp.row0 + i0 + tk) * p.heads + a) * p.vdim + col] = o;
         }
     }
     if (!live) return;
 #pragma unroll
     for (int n = 0; n < RP; ++n) {
-        const uint32_t i = part * RP + n;
+        const uint32_t i = part + 16 * n;
         if (i < p.dim) state[(size_t)i * p.vdim + col] = S[n];
     }
 }
@@ -112,14 +142,14 @@ uzu_status channel_delta(hipStream_t s, const ChannelDeltaParams& p) {
     if (!p.rows) return UZU_OK;
     UZU_REQUIRE(p.qkv && p.decay && p.beta && p.out && p.states && p.spans && p.nseq && p.heads && p.groups && p.heads % p.groups == 0, "channel_delta: null argument");
     UZU_UNSUPPORTED(!channel_delta_supported(p.dim, p.vdim), "channel_delta: heads of %u x %u (keys up to 256)", p.dim, p.vdim);
-    UZU_REQUIRE((size_t)p.nseq * p.heads <= 0x7FFFFFFFu && (p.vdim + 63) / 64 <= 65535, "channel_delta: too many heads for one launch");
-    const dim3 grid(p.nseq * p.heads, (p.vdim + 63) / 64);
+    UZU_REQUIRE((size_t)p.nseq * p.heads <= 0x7FFFFFFFu && (p.vdim + 15) / 16 <= 65535, "channel_delta: too many heads for one launch");
+    const dim3 grid(p.nseq * p.heads, (p.vdim + 15) / 16);
 #define UZU_CD(RP) return launch_check([&] { hipLaunchKernelGGL((channel_delta_steps_kernel<RP>), grid, dim3(256), 0, s, p); }, "channel_delta_steps")
-    if (p.dim <= 16) UZU_CD(4);
-    if (p.dim <= 32) UZU_CD(8);
-    if (p.dim <= 64) UZU_CD(16);
-    if (p.dim <= 128) UZU_CD(32);
-    UZU_CD(64);
+    if (p.dim <= 16) UZU_CD(1);
+    if (p.dim <= 32) UZU_CD(2);
+    if (p.dim <= 64) UZU_CD(4);
+    if (p.dim <= 128) UZU_CD(8);
+    UZU_CD(16);
 #undef UZU_CD
 }
 

@@ -632,7 +632,15 @@ class ModelBundle:
         for l in self.layers:
             if l.mixer_kind == MIXER_ATTENTION:
                 rows = min(context, l.sliding_window_size) if l.sliding_window_size else context
+                if l.attention_chunk_size:  # at most the row's own chunk
+                    rows = min(rows, l.attention_chunk_size)
                 total += rows * l.num_groups * (l.head_dim + (l.value_head_dim or l.head_dim)) * 2  # K and V rows, bf16 (a sharing layer reads its source's)
+                if l.pair_mixer is not None:  # the delta rule beside it: f32 state read + write, the convolution's window and taps
+                    total += 2 * l.dn_num_heads * l.dn_value_head_dim * l.dn_head_dim * 4
+                    conv_dim = 2 * l.dn_num_groups * l.dn_head_dim + l.dn_num_heads * l.dn_value_head_dim
+                    total += conv_dim * (3 * l.dn_kernel_size - 2) * 4
+                if l.input_conv_taps:  # the sublayers' input convolutions: window read + write, taps
+                    total += 2 * self.model_dim * (3 * l.input_conv_taps - 2) * 4
             elif l.mixer_kind == MIXER_RETENTION:
                 total += 2 * l.num_heads * l.head_dim * l.value_head_dim * 4  # f32 state read + write
             elif l.mixer_kind == MIXER_LATENT_ATTENTION:
@@ -666,7 +674,11 @@ class ModelBundle:
             if l.mixer_kind == MIXER_ATTENTION and l.value_head_dim:  # an f32-stream design's attention: its own value width, the window counted
                 w = l.sliding_window_size
                 vis = pairs if not w else min(pairs, tokens * float(w))
+                if l.attention_chunk_size:  # a row sees (chunk + 1) / 2 keys of its own chunk on average
+                    vis = min(vis, tokens * (l.attention_chunk_size + 1) / 2.0)
                 flops += 2.0 * vis * l.num_heads * (l.head_dim + l.value_head_dim)
+                if l.pair_mixer is not None:  # the delta rule beside it: ~6 flops per state element per token (decay, S k, rank-1 update, S q)
+                    flops += 6.0 * tokens * l.dn_num_heads * l.dn_value_head_dim * l.dn_head_dim
             elif l.mixer_kind == MIXER_ATTENTION:
                 flops += 4.0 * pairs * l.num_heads * l.head_dim
             elif l.mixer_kind == MIXER_RETENTION:  # per token and head: the outer-product update and the read-out of the state

@@ -225,19 +225,19 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
     for (uint32_t c : counts) rows += c;
     const size_t slot_stride = (size_t)S.max_rows * d;
     const uint32_t bf = S.full_f32 ? 0u : 1u;
+    uint32_t max_count = 0;
+    for (uint32_t c : counts) max_count = std::max(max_count, c);
     if (S.pair_table) { // + the hashed (previous token, token) row; two launches: the rows, then the sequences' new previous tokens
         k::EmbedPairParams ep{};
         ep.tokens = d_tokens, ep.table = (const uint16_t*)m->embedding.w, ep.pair_table = S.pair_table, ep.out = S.slots, ep.rows = rows, ep.vocab = m->d.vocab_size, ep.d = d;
         ep.scale = m->d.input_scale, ep.buckets = m->d.bigram_buckets, ep.mul_prev = m->d.bigram_mul_prev, ep.mul_cur = m->d.bigram_mul_cur, ep.spans = S.d_spans;
-        ep.row_seq = S.d_row_seq, ep.prev = S.d_prev_tok_ptrs, ep.nseq = nseq;
+        ep.row_seq = S.d_row_seq, ep.prev = S.d_prev_tok_ptrs, ep.nseq = nseq, ep.max_count = max_count;
         RUN("embed_pair_rows_f32", (size_t)rows * d * 8, k::embed_pair_rows_f32(s, ep));
-        ++m->launches;
+        if (max_count > 1) ++m->launches;
     } else {
         RUN("embed_rows_f32", (size_t)rows * d * 6, k::embed_rows_f32(s, d_tokens, (const uint16_t*)m->embedding.w, S.slots, rows, m->d.vocab_size, d, m->d.input_scale));
     }
     const float* cur = S.slots; // what the layer about to run reads: X_0, then the depth mix of the layer before
-    uint32_t max_count = 0;
-    for (uint32_t c : counts) max_count = std::max(max_count, c);
     // A sublayer's result joins the stream behind its post norm; the same launch leaves the norm of the new rows for the sublayer that follows where that is an
     // RMS norm with a weight vector (`next`), so that norm needs no launch of its own.
     auto add_normed = [&](const float* y, const float* residual, float* out, const DNorm& N, const float* layer_scale, const DNorm* next) {
@@ -252,8 +252,9 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
         k::CausalConvParams cp{};
         cp.x = x, cp.ldx = d, cp.out = S.normed, cp.ldo = d, cp.w = w, cp.channels = d, cp.taps = taps, cp.add_input = 1;
         cp.states = S.d_inconv_ptrs + (size_t)l * S.max_seqs, cp.state_offset = (size_t)which * (taps - 1) * d, cp.spans = S.d_spans, cp.row_seq = S.d_row_seq, cp.nseq = nseq, cp.rows = rows;
+        cp.max_count = max_count;
         RUN("causal_conv_rows", (size_t)rows * d * 4 * (taps + 1), k::causal_conv_rows(s, cp));
-        if (taps > 1) RUN("causal_conv_commit", (size_t)nseq * d * 8 * (taps - 1), k::causal_conv_commit(s, cp));
+        if (taps > 1 && max_count > 1) RUN("causal_conv_commit", (size_t)nseq * d * 8 * (taps - 1), k::causal_conv_commit(s, cp));
         return S.normed;
     };
     bool normed_ready = false; // S.normed already holds this run's pre-mixer norm (left by the run before)
@@ -406,9 +407,9 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             run_linear(e, lin(S, L.in_proj, mix_in, S.dn_in, rows)); // q | k | v | beta | decay down | gate down
             k::CausalConvParams cp{};
             cp.x = S.dn_in, cp.ldx = ldi, cp.out = S.dn_cv, cp.ldo = conv_dim, cp.w = L.conv_w, cp.bias = L.conv_b, cp.channels = conv_dim, cp.taps = taps, cp.act = 1;
-            cp.states = S.d_pair_conv_ptrs + (size_t)l * S.max_seqs, cp.spans = S.d_spans, cp.row_seq = S.d_row_seq, cp.nseq = nseq, cp.rows = rows;
+            cp.states = S.d_pair_conv_ptrs + (size_t)l * S.max_seqs, cp.spans = S.d_spans, cp.row_seq = S.d_row_seq, cp.nseq = nseq, cp.rows = rows, cp.max_count = max_count;
             RUN("causal_conv_rows", (size_t)rows * conv_dim * 4 * (taps + 1), k::causal_conv_rows(s, cp));
-            if (taps > 1) RUN("causal_conv_commit", (size_t)nseq * conv_dim * 8 * (taps - 1), k::causal_conv_commit(s, cp));
+            if (taps > 1 && max_count > 1) RUN("causal_conv_commit", (size_t)nseq * conv_dim * 8 * (taps - 1), k::causal_conv_commit(s, cp));
             {   // the low-rank factors' second halves: what enters the recurrence is never rounded, true f32 products in both precisions
                 k::LinearF32Params up = lin(S, X.decay_up, S.dn_in + a_col, S.dn_decay, rows);
                 up.ldx = ldi, up.bf16_products = 0;

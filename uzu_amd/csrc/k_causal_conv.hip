@@ -13,7 +13,19 @@ namespace k {
 
 namespace {
 
-// thread = (row, channel)
+// the inputs of positions end - (taps - 1) .. end - 1 of sequence z, channel c: from this pass's rows, the old window, or (in front of position 0) zeros
+__device__ __forceinline__ void window_update(const CausalConvParams& p, const SeqSpan& sp, uint32_t z, uint32_t c) {
+    float* cs = p.states[z] + p.state_offset;
+    const uint32_t keep = p.taps - 1;
+    for (uint32_t s = 0; s < keep; ++s) { // ascending: an old entry is read at index s + count > s before that index is written
+        float v = 0.0f;
+        if (s + sp.count >= keep) v = p.x[(size_t)(sp.row0 + (s + sp.count - keep)) * p.ldx + p.x_col + c];
+        else if (sp.start + sp.count + s >= keep) v = cs[(size_t)(s + sp.count) * p.channels + c];
+        cs[(size_t)s * p.channels + c] = v;
+    }
+}
+
+// thread = (row, channel).  A sequence that brings ONE row (a decode step) has its window replaced here: the row's own thread is the only reader of the old one.
 __global__ void __launch_bounds__(256) causal_conv_rows_kernel(CausalConvParams p) {
     const uint32_t r = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
     if (c >= p.channels) return;
@@ -34,21 +46,16 @@ __global__ void __launch_bounds__(256) causal_conv_rows_kernel(CausalConvParams 
     if (p.act == 1) acc = acc / (1.0f + expf(-acc));
     if (p.add_input) acc = own + acc;
     p.out[(size_t)r * p.ldo + p.o_col + c] = acc;
+    if (sp.count == 1 && p.taps > 1) window_update(p, sp, z, c);
 }
 
-// thread = (sequence, channel): the inputs of positions end - (taps - 1) .. end - 1, from this pass's rows, the old state, or (in front of position 0) zeros
+// thread = (sequence, channel): the windows of the sequences that bring several rows (their first rows' threads read the old window in the launch before)
 __global__ void __launch_bounds__(256) causal_conv_commit_kernel(CausalConvParams p) {
     const uint32_t z = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
     if (c >= p.channels) return;
     const SeqSpan sp = p.spans[z];
-    float* cs = p.states[z] + p.state_offset;
-    const uint32_t keep = p.taps - 1;
-    for (uint32_t s = 0; s < keep; ++s) { // ascending: an old entry is read at index s + count > s before that index is written
-        float v = 0.0f;
-        if (s + sp.count >= keep) v = p.x[(size_t)(sp.row0 + (s + sp.count - keep)) * p.ldx + p.x_col + c];
-        else if (sp.start + sp.count + s >= keep) v = cs[(size_t)(s + sp.count) * p.channels + c];
-        cs[(size_t)s * p.channels + c] = v;
-    }
+    if (sp.count == 1) return; // done by the row's own thread
+    window_update(p, sp, z, c);
 }
 
 // a wave per (row, head): x / sqrt(mean(x^2) + eps) * weight * gate
@@ -81,7 +88,7 @@ uzu_status causal_conv_rows(hipStream_t s, const CausalConvParams& p) {
 }
 
 uzu_status causal_conv_commit(hipStream_t s, const CausalConvParams& p) {
-    if (!p.rows || p.taps < 2) return UZU_OK;
+    if (!p.rows || p.taps < 2 || p.max_count == 1) return UZU_OK; // (every sequence brings one row: the rows' launch has replaced the windows)
     UZU_REQUIRE(p.x && p.states && p.spans && p.nseq && p.channels, "causal_conv: null argument");
     return launch_check([&] { hipLaunchKernelGGL(causal_conv_commit_kernel, dim3(p.nseq, (p.channels + 255) / 256), dim3(256), 0, s, p); }, "causal_conv_commit");
 }

@@ -38,12 +38,24 @@ __global__ void __launch_bounds__(256) channel_delta_prep_kernel(ChannelDeltaPar
 
 constexpr int kStage = 16; // tokens whose q / k / decay / v / beta are staged at once
 
+// the sum over the 16 lanes of a row of the wave, left in every one of them: four data-parallel-primitive moves (quad swaps, then the two mirrors) -- the same
+// order in every launch
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // quad_perm [1, 0, 3, 2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // quad_perm [2, 3, 0, 1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true)); // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true)); // row_mirror
+    return v;
+}
+
 // grid (sequence * heads, ceil(dv / 16)); thread = (column, sixteenth of the rows): a wave owns 4 columns, a workgroup 16.  RP = rows per thread (dk <= 16 RP);
-// thread `part` of a column owns rows part, part + 16, ...  The next stage's rows travel from memory into registers while the current stage is worked on.
+// thread `part` of a column owns rows part * RP .. part * RP + RP - 1, which lie side by side in LDS (16-byte reads; a pad of four floats per part keeps the
+// sixteen parts on different banks).  The next stage's rows travel from memory into registers while the current stage is worked on.
 template <int RP>
 __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaParams p) {
-    constexpr int DK = 16 * RP;
-    __shared__ float s_k[kStage][DK], s_q[kStage][DK], s_g[kStage][DK], s_v[kStage][16], s_b[kStage];
+    constexpr int DK = 16 * RP, PW = RP >= 8 ? RP + 4 : RP, LDW = 16 * PW;
+    __shared__ __attribute__((aligned(16))) float s_k[kStage][LDW], s_q[kStage][LDW], s_g[kStage][LDW];
+    __shared__ float s_v[kStage][16], s_b[kStage];
     const uint32_t z = blockIdx.x / p.heads, a = blockIdx.x % p.heads, g = a / (p.heads / p.groups);
     const uint32_t tid = threadIdx.x, cl = tid >> 4, part = tid & 15, col = blockIdx.y * 16 + cl;
     const bool live = col < p.vdim;
@@ -52,7 +64,7 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
     float S[RP];
 #pragma unroll
     for (int n = 0; n < RP; ++n) {
-        const uint32_t i = part + 16 * n;
+        const uint32_t i = part * RP + n;
         S[n] = (sp.start && live && i < p.dim) ? state[(size_t)i * p.vdim + col] : 0.0f;
     }
     float pf[3 * RP], pf_v = 0.0f, pf_b = 0.0f;
@@ -81,7 +93,7 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
         for (int e = 0; e < 3 * RP; ++e) {
             const uint32_t rem = (uint32_t)(e % RP) * 256 + tid, tk = rem / DK, i = rem % DK;
             float* dst = e / RP == 0 ? &s_k[0][0] : e / RP == 1 ? &s_q[0][0] : &s_g[0][0];
-            dst[tk * DK + i] = pf[e];
+            dst[tk * LDW + (i / RP) * PW + i % RP] = pf[e];
         }
         s_v[tid >> 4][tid & 15] = pf_v;
         if (tid < (uint32_t)kStage) s_b[tid] = pf_b;
@@ -95,35 +107,41 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
         if (i0 + kStage < sp.count) fetch(i0 + kStage);
         for (uint32_t tk = 0; tk < nt; ++tk) {
             const float v = s_v[tk][cl], beta = s_b[tk];
-            const float *kk = &s_k[tk][part], *qq = &s_q[tk][part], *gg = &s_g[tk][part];
+            float kk[RP], qq[RP], gg[RP];
+            if constexpr (RP % 4 == 0) {
+#pragma unroll
+                for (int n = 0; n < RP; n += 4) {
+                    const f32x4_v k4 = *(const f32x4_v*)&s_k[tk][part * PW + n], q4 = *(const f32x4_v*)&s_q[tk][part * PW + n], g4 = *(const f32x4_v*)&s_g[tk][part * PW + n];
+                    kk[n] = k4.x, kk[n + 1] = k4.y, kk[n + 2] = k4.z, kk[n + 3] = k4.w;
+                    qq[n] = q4.x, qq[n + 1] = q4.y, qq[n + 2] = q4.z, qq[n + 3] = q4.w;
+                    gg[n] = g4.x, gg[n + 1] = g4.y, gg[n + 2] = g4.z, gg[n + 3] = g4.w;
+                }
+            } else {
+#pragma unroll
+                for (int n = 0; n < RP; ++n) kk[n] = s_k[tk][part * PW + n], qq[n] = s_q[tk][part * PW + n], gg[n] = s_g[tk][part * PW + n];
+            }
             float dot = 0.0f;
 #pragma unroll
             for (int n = 0; n < RP; ++n) {
-                S[n] *= gg[16 * n];
-                dot = fmaf(S[n], kk[16 * n], dot);
+                S[n] *= gg[n];
+                dot = fmaf(S[n], kk[n], dot);
             }
-            dot += __shfl_xor(dot, 1, 64);
-            dot += __shfl_xor(dot, 2, 64);
-            dot += __shfl_xor(dot, 4, 64);
-            dot += __shfl_xor(dot, 8, 64);
+            dot = row16_sum(dot);
             const float u = beta * (v - dot);
             float o = 0.0f;
 #pragma unroll
             for (int n = 0; n < RP; ++n) {
-                S[n] = fmaf(kk[16 * n], u, S[n]);
-                o = fmaf(S[n], qq[16 * n], o);
+                S[n] = fmaf(kk[n], u, S[n]);
+                o = fmaf(S[n], qq[n], o);
             }
-            o += __shfl_xor(o, 1, 64);
-            o += __shfl_xor(o, 2, 64);
-            o += __shfl_xor(o, 4, 64);
-            o += __shfl_xor(o, 8, 64);
+            o = row16_sum(o);
             if (live && part == 0) p.out[((size_t)(sp.row0 + i0 + tk) * p.heads + a) * p.vdim + col] = o;
         }
     }
     if (!live) return;
 #pragma unroll
     for (int n = 0; n < RP; ++n) {
-        const uint32_t i = part + 16 * n;
+        const uint32_t i = part * RP + n;
         if (i < p.dim) state[(size_t)i * p.vdim + col] = S[n];
     }
 }

@@ -65,13 +65,14 @@ __global__ void __launch_bounds__(256) embed_pair_rows_f32_kernel(EmbedPairParam
     const uint16_t* add = p.pair_table + (size_t)row * p.d;
     float* dst = p.out + (size_t)r * p.d;
     for (uint32_t c = threadIdx.x; c < p.d; c += blockDim.x) dst[c] = bf16_to_f32(src[c]) * p.scale + bf16_to_f32(add[c]);
+    if (sp.count == 1 && threadIdx.x == 0) *p.prev[z] = p.tokens[r]; // a sequence that brings one row: this workgroup is the only reader of the old token
 }
 // thread = sequence: its last token of the pass becomes the state's previous token (a launch of its own: the rows above read the old one)
 __global__ void __launch_bounds__(64) embed_pair_commit_kernel(EmbedPairParams p, uint32_t nseq) {
     const uint32_t z = blockIdx.x * 64 + threadIdx.x;
     if (z >= nseq) return;
     const SeqSpan sp = p.spans[z];
-    *p.prev[z] = p.tokens[sp.row0 + sp.count - 1];
+    if (sp.count > 1) *p.prev[z] = p.tokens[sp.row0 + sp.count - 1];
 }
 
 constexpr int kNormUnroll = 8;
@@ -588,6 +589,7 @@ uzu_status embed_pair_rows_f32(hipStream_t s, const EmbedPairParams& p) {
     if (!p.rows) return UZU_OK;
     UZU_REQUIRE(p.tokens && p.table && p.pair_table && p.out && p.spans && p.row_seq && p.prev && p.buckets && p.nseq, "embed_pair_rows_f32: null argument");
     UZU_PROPAGATE(launch_check([&] { hipLaunchKernelGGL(embed_pair_rows_f32_kernel, dim3(p.rows), dim3(256), 0, s, p); }, "embed_pair_rows_f32"));
+    if (p.max_count == 1) return UZU_OK;
     return launch_check([&] { hipLaunchKernelGGL(embed_pair_commit_kernel, dim3((p.nseq + 63) / 64), dim3(64), 0, s, p, p.nseq); }, "embed_pair_commit");
 }
 

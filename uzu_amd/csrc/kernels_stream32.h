@@ -48,7 +48,7 @@ struct EmbedPairParams {
     const SeqSpan* spans;
     const uint32_t* row_seq;
     uint32_t* const* prev; // device array [nseq] of device pointers
-    uint32_t nseq;
+    uint32_t nseq, max_count; // max_count (the longest share of the pass, 0 = unknown) == 1: no second launch, the row's own workgroup stores the token
 };
 uzu_status embed_pair_rows_f32(hipStream_t s, const EmbedPairParams& p);
 
@@ -353,7 +353,8 @@ uzu_status lru_scan(hipStream_t s, const GatedLruParams& p);
 // xin = channel c of the sequence's input rows `x` (f32, pitch ldx, column x_col): of this pass, or (in front of the pass) the taps - 1 inputs the state keeps
 // (states[z] + state_offset: f32 [taps - 1][channels], oldest first), or zero in front of position 0.  w f32 [channels][taps]: the last tap weighs the row itself.
 // act: 0 none, 1 silu.  `out` is another block of rows than `x`.  causal_conv_commit leaves the last taps - 1 inputs behind the pass in the state; it reads the
-// same `x`, which must still hold the pass's inputs.
+// same `x`, which must still hold the pass's inputs.  A sequence that brings one row has its window replaced by causal_conv_rows itself; max_count (the longest
+// share of the pass, 0 = unknown) == 1 makes causal_conv_commit a no-op.
 struct CausalConvParams {
     const float* x;
     uint32_t ldx, x_col;
@@ -365,7 +366,7 @@ struct CausalConvParams {
     size_t state_offset;  // floats
     const SeqSpan* spans;
     const uint32_t* row_seq;
-    uint32_t nseq, rows;
+    uint32_t nseq, rows, max_count;
 };
 uzu_status causal_conv_rows(hipStream_t s, const CausalConvParams& p);
 uzu_status causal_conv_commit(hipStream_t s, const CausalConvParams& p);

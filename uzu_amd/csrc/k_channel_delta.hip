@@ -105,7 +105,9 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
         put();
         __syncthreads();
         if (i0 + kStage < sp.count) fetch(i0 + kStage);
-        for (uint32_t tk = 0; tk < nt; ++tk) {
+        // one token: only  S -> decayed S -> <S, k> -> u -> S  is the recurrence; the read-out <S, q> of a token overlaps the next token's chain when a full stage
+        // is unrolled.  The dot products are sums of four interleaved partial sums (rows n = 0, 4, .. | 1, 5, .. | ..), then of the sixteen threads: a fixed order.
+        auto step = [&](uint32_t tk) {
             const float v = s_v[tk][cl], beta = s_b[tk];
             float kk[RP], qq[RP], gg[RP];
             if constexpr (RP % 4 == 0) {
@@ -120,22 +122,28 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
 #pragma unroll
                 for (int n = 0; n < RP; ++n) kk[n] = s_k[tk][part * PW + n], qq[n] = s_q[tk][part * PW + n], gg[n] = s_g[tk][part * PW + n];
             }
-            float dot = 0.0f;
+            float d[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int n = 0; n < RP; ++n) {
                 S[n] *= gg[n];
-                dot = fmaf(S[n], kk[n], dot);
+                d[n & 3] = fmaf(S[n], kk[n], d[n & 3]);
             }
-            dot = row16_sum(dot);
+            const float dot = row16_sum((d[0] + d[1]) + (d[2] + d[3]));
             const float u = beta * (v - dot);
-            float o = 0.0f;
+            float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int n = 0; n < RP; ++n) {
                 S[n] = fmaf(kk[n], u, S[n]);
-                o = fmaf(S[n], qq[n], o);
+                o[n & 3] = fmaf(S[n], qq[n], o[n & 3]);
             }
-            o = row16_sum(o);
-            if (live && part == 0) p.out[((size_t)(sp.row0 + i0 + tk) * p.heads + a) * p.vdim + col] = o;
+            const float out = row16_sum((o[0] + o[1]) + (o[2] + o[3]));
+            if (live && part == 0) p.out[((size_t)(sp.row0 + i0 + tk) * p.heads + a) * p.vdim + col] = out;
+        };
+        if (nt == (uint32_t)kStage) {
+#pragma unroll
+            for (int tk = 0; tk < kStage; ++tk) step(tk);
+        } else {
+            for (uint32_t tk = 0; tk < nt; ++tk) step(tk);
         }
     }
     if (!live) return;

@@ -129,6 +129,9 @@ def test_reader_maps_every_branch_of_the_schema(tmp_path):
     assert a.qkv_projection.n == 6 * 4 + 3 * 4 + 3 * 8 + 6 and a.query_norm.scales.shape == (24,) and a.key_norm.scales.shape == (12,) and a.sinks.shape == (6,)
     assert a.no_mlp and a.input_conv_mlp is None and a.attention_scale == pytest.approx(0.7) and not a.attention_chunk_size and not a.values_are_keys
     assert b.ropes[a.rope_index].head_dim == 2 and b.ropes[a.rope_index].base == 500.0 and not c.use_rope and len(b.ropes) == 1
+    spare = dict(W)  # a layer without a dense block whose file still carries the second sublayer's norm and convolution: read, not used
+    spare["l1.norm2"], spare["l1.canon2"] = W["l1.norm1"], W["l1.canon1"]
+    assert loader.load_model_dir(write(tmp_path, cfg, spare, "spare"), max_context_length=64).layers[1].no_mlp
     d = b.desc()  # the ctypes description carries them
     assert d.bigram_buckets == 19 and d.layers[0].pair_mixer == 1 + D.MIXER_DELTA_NET and d.layers[0].rel_bias_rows == 7 and d.layers[1].qk_norm_whole == 1
     assert d.layers[0].dn_decay_rank == 3 and d.output_norm.groups == 3 and d.logit_soft_cap == 8.0

@@ -135,6 +135,9 @@ def load(path: str, cfg: dict, st, max_context_length: Optional[int], name: Opti
         ml = lc.get("mlp")
         if ml is None:
             lw.no_mlp = True
+            for spare in (p + "norm2", p + "canon2"):  # a layer without a dense block has no use for them; a file that carries them all the same is read
+                if t.has(spare):
+                    st.consumed.add(spare)
         elif ml.get("kind") == "dense":
             ff = int(ml.get("ff") or t.shape(p + "mlp.gate")[0])
             lw.hidden_dim = ff

@@ -166,8 +166,8 @@ def test_unequal_batch_equals_each_request_alone_and_reused_states(models, name)
         alone.append(np.concatenate([first] + tail))
         st.close()
     pool = [m.new_state() for _ in reqs]
-    for round_ in range(2):  # the second round reuses the states the first one gave back (reset), in another order: caches, recurrent states, windows and previous tokens of other requests
-        states = pool if round_ == 0 else pool[::-1]
+    for turn in range(2):  # the second turn reuses the states the first one gave back (reset), in another order: caches, recurrent states, windows and previous tokens of other requests
+        states = pool if turn == 0 else pool[::-1]
         heads = [r[:-3] if len(r) > 3 else r for r in reqs]
         lg, _ = m.step_batch(states, heads, [[len(h) - 1] for h in heads])
         got = [[lg[i]] for i in range(len(reqs))]
@@ -177,7 +177,7 @@ def test_unequal_batch_equals_each_request_alone_and_reused_states(models, name)
             for row, i in zip(lg, live):
                 got[i].append(row)
         for i in range(len(reqs)):
-            assert np.abs(np.stack(got[i]) - alone[i]).max() < 2e-4 * np.abs(alone[i]).max(), (round_, i)
+            assert np.abs(np.stack(got[i]) - alone[i]).max() < 2e-4 * np.abs(alone[i]).max(), (turn, i)
             assert O.logit_error(np.stack(got[i])[-1:], O.forward(cfg, W, reqs[i])[0][-1:]).max() < TOL[True]
         for st in states:
             st.reset()
@@ -381,7 +381,7 @@ def test_greedy_generation_through_prefill_and_decode(models, name):
 
 def test_generate_loop_of_the_text_front_end_and_the_pool(hip_ctx, tmp_path):
     """LanguageModel.generate on a directory without tokenizer.json, and SequencePool.generate: prompts of unequal length prefilled in one batch and decoded
-    together, requests leaving as they finish (one by a stop token), their states reused by a second round -- against each prompt generated alone by the oracle"""
+    together, requests leaving as they finish (one by a stop token), their states reused by a second call -- against each prompt generated alone by the oracle"""
     from uzu_amd.language_model import LanguageModel
     from uzu_amd.serving import SequencePool
     cfg = cfg_a()

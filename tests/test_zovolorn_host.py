@@ -1,5 +1,5 @@
 """Zovolorn on the host: identities of the float64 oracle (what the GPU tests lean on), and the config.json reader -- every branch of the schema, the engine
-description it produces (packed projections, the second mixer's fields, absent pre norms), its refusals, and the writer's round trip.  No GPU."""
+description it produces (packed projections, the second mixer's fields, absent pre norms), its refusals, and what the writer writes read back.  No GPU."""
 import json
 import os
 
@@ -174,7 +174,7 @@ def test_reader_refusals(tmp_path):
             loader.load_model_dir(broken(change, f"bad{i}"), max_context_length=64)
 
 
-def test_writer_round_trip(tmp_path):
+def test_what_the_writer_writes_reads_back(tmp_path):
     cfg = zovolorn.config(37, 16, [
         zovolorn.parallel_layer(2, 1, 8, 12, 6, 30.0, 2, 1, 4, 8, 3, rank=2, left_scale=0.6, right_scale=0.9, mlp=zovolorn.dense_mlp(8)),
         zovolorn.attention_layer(2, 1, 8, 4, rot_dims=4, mlp=None)], groups=2, taps=2, embed_scale=0.25, bigram=(11, 3, 2), logit_softcap=5.0)

@@ -106,6 +106,7 @@ MECHANISMS = {
     "delta_rule_three_heads_per_group_odd_widths": one_layer(pair(d_heads=6, d_kv_heads=2, d_dim=5, d_vdim=7, conv=2, left_scale=0.0)),
     "delta_rule_wide": one_layer(pair(d_heads=1, d_kv_heads=1, d_dim=33, d_vdim=70, conv=4, rank=9, left_scale=0.0)),
     "delta_rule_keys_of_130": one_layer(pair(d_heads=2, d_kv_heads=2, d_dim=130, d_vdim=4, conv=1, left_scale=0.0)),
+    "delta_rule_keys_of_100": one_layer(pair(d_heads=2, d_kv_heads=1, d_dim=100, d_vdim=20, conv=3, left_scale=0.0)),
     "pair_with_dense_block": one_layer(pair(mlp=O.dense(24), left_scale=0.6, right_scale=0.9)),
     "one_tap": one_layer(O.attention_layer(2, 1, 8, 8, rot_dims=4, mlp=O.dense(16)), taps=1),
     "five_taps": one_layer(O.attention_layer(2, 1, 8, 8, rot_dims=4, mlp=O.dense(16)), taps=5),
@@ -130,6 +131,25 @@ def test_each_mechanism_alone_in_a_one_layer_model(hip_ctx, tmp_path, which):
     st.reset()  # and token by token from a reused state: the decode forms of the same kernels
     rows = [m.step_batch([st], [[t]], [[0]])[0][0] for t in toks[:40]]
     assert O.logit_error(np.stack(rows), want[:40]).max() < TOL[True]
+    st.close()
+    m.close()
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_heads_of_128_in_both_precisions(hip_ctx, tmp_path, full):
+    """Head widths of real models: the serving precision runs the attention on the matrix cores over bf16 caches (chunks, distance bias, temperatures, sinks and
+    gates inside that form), the delta rule holds eight rows per thread; prompt rows, a portion across a chunk's edge and decoded tokens against the oracle."""
+    cfg = O.config(vocab=97, width=64, groups=2, taps=3, bigram=(53, 3, 7), layers=[
+        O.parallel_layer(2, 1, 128, 48, 16, 100.0, 2, 1, 128, 128, 3, rank=8, scale=0.09, left_scale=0.6, right_scale=0.9, mlp=None),
+        O.attention_layer(2, 1, 128, 128, rot_dims=64, rot_base=5e5, scale=0.09, mlp=O.dense(32))])
+    W, m = make(hip_ctx, tmp_path, cfg, 13, flags=MODEL_FULL_F32 if full else 0)
+    toks = prompt(cfg, 140, 4)
+    want, _ = O.forward(cfg, W, toks)
+    st = m.new_state()
+    a, _ = m.step_batch([st], [toks[:90]], [list(range(90))])
+    b, _ = m.step_batch([st], [toks[90:120]], [list(range(30))])
+    tail = [m.step_batch([st], [[t]], [[0]])[0][0] for t in toks[120:]]
+    assert rows_ok(O.logit_error(np.concatenate([a, b, np.stack(tail)]), want), full)
     st.close()
     m.close()
 

@@ -55,7 +55,7 @@ template <int RP>
 __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaParams p) {
     constexpr int DK = 16 * RP, PW = RP >= 8 ? RP + 4 : RP, LDW = 16 * PW;
     __shared__ __attribute__((aligned(16))) float s_k[kStage][LDW], s_q[kStage][LDW], s_g[kStage][LDW];
-    __shared__ float s_v[kStage][16], s_b[kStage];
+    __shared__ float s_v[kStage][16], s_b[kStage], s_o[kStage][16];
     const uint32_t z = blockIdx.x / p.heads, a = blockIdx.x % p.heads, g = a / (p.heads / p.groups);
     const uint32_t tid = threadIdx.x, cl = tid >> 4, part = tid & 15, col = blockIdx.y * 16 + cl;
     const bool live = col < p.vdim;
@@ -98,10 +98,16 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
         s_v[tid >> 4][tid & 15] = pf_v;
         if (tid < (uint32_t)kStage) s_b[tid] = pf_b;
     };
+    // a stage's results leave through LDS, one coalesced store per thread (a store per token and column from inside the chain costs 40 % of the launch)
+    auto flush = [&](uint32_t i0, uint32_t nt) {
+        const uint32_t tk = tid >> 4, c = blockIdx.y * 16 + (tid & 15);
+        if (tk < nt && c < p.vdim) p.out[((size_t)(sp.row0 + i0 + tk) * p.heads + a) * p.vdim + c] = s_o[tk][tid & 15];
+    };
     fetch(0);
     for (uint32_t i0 = 0; i0 < sp.count; i0 += kStage) {
         const uint32_t nt = sp.count - i0 < (uint32_t)kStage ? sp.count - i0 : (uint32_t)kStage;
-        __syncthreads(); // the stage before has been read
+        __syncthreads(); // the stage before has been read, its results stand in s_o
+        if (i0) flush(i0 - kStage, kStage);
         put();
         __syncthreads();
         if (i0 + kStage < sp.count) fetch(i0 + kStage);
@@ -137,7 +143,7 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
                 o[n & 3] = fmaf(S[n], qq[n], o[n & 3]);
             }
             const float out = row16_sum((o[0] + o[1]) + (o[2] + o[3]));
-            if (live && part == 0) p.out[((size_t)(sp.row0 + i0 + tk) * p.heads + a) * p.vdim + col] = out;
+            if (part == 0) s_o[tk][cl] = out;
         };
         if (nt == (uint32_t)kStage) {
 #pragma unroll
@@ -145,6 +151,11 @@ __global__ void __launch_bounds__(256) channel_delta_steps_kernel(ChannelDeltaPa
         } else {
             for (uint32_t tk = 0; tk < nt; ++tk) step(tk);
         }
+    }
+    __syncthreads();
+    {
+        const uint32_t last = (sp.count - 1) / kStage * kStage;
+        flush(last, sp.count - last);
     }
     if (!live) return;
 #pragma unroll

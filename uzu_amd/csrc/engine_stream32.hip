@@ -58,6 +58,10 @@ struct Stream32 {
     uint32_t** d_prev_tok_ptrs = nullptr; // [max_seqs]: the previous token (hashed token-pair table)
     float *dn_in = nullptr, *dn_cv = nullptr, *dn_decay = nullptr, *dn_gate = nullptr, *dn_o = nullptr; // the delta rule: packed projection, convolved q | k | v, decays, gate, result
     uint16_t* pair_table = nullptr; // bf16 [buckets + 1][d]
+    // a pair of mixers in a prompt-sized pass: the first mixer's launches run on a stream of their own beside the second's (its recurrence is a chain of dependent
+    // steps on few workgroups and leaves most of the chip idle); default priority, joined again in front of the out projections
+    hipStream_t side = nullptr;
+    hipEvent_t side_fork = nullptr, side_join = nullptr;
     struct Layer {
         uint16_t* up_keys_t = nullptr; // bf16 [heads][rank][head_dim]: W_up_k of a head transposed, so that folding it into the query is an ordinary product
         float* sinks = nullptr;        // f32 [heads]
@@ -216,7 +220,8 @@ uzu_status s32_upload_tables(uzu_hip_model* m, const std::vector<PassSeq>& seqs,
 // device-side spans -- so a one-token step can be captured once and replayed.  Does not move the sequences' context lengths.
 uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, const uint32_t* d_tokens, uint32_t n_out) {
     Stream32& S = *m->s32;
-    hipStream_t s = m->ctx->stream;
+    hipStream_t s = m->ctx->stream; // (the stream the next launch goes to: a pair's first mixer switches it to S.side and back)
+    const hipStream_t main_stream = s;
     Enc e{m, s};
     e.prof = (std::vector<ProfEntry>*)m->prof_sink;
     m->launches = 0;
@@ -294,6 +299,15 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             RUN("dyn_tanh_norm+shift", (size_t)rows * d * 8, k::dyn_tanh_norm(s, np));
         }
         const uint32_t H = h.num_heads, hd = h.head_dim, vd = h.value_head_dim, rank = h.latent_rank;
+        // prompt-sized pass over a pair of mixers: the first one's projection, rotation / append and attention core go to the side stream (they touch S.q, S.attn and
+        // the caches; the second mixer touches its own rows); not while a launch is being timed or captured
+        bool forked = false;
+        if (h.pair_mixer && S.side && rows >= 256 && !e.prof) {
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(main_stream, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone && hipEventRecord(S.side_fork, main_stream) == hipSuccess &&
+                hipStreamWaitEvent(S.side, S.side_fork, 0) == hipSuccess)
+                forked = true, s = S.side, e.s = S.side;
+        }
         run_linear(e, lin(S, L.qkv, mix_in, S.q, rows)); // the packed projection of the mixer (queries first)
         if (h.mixer_kind == UZU_MIXER_GATED_LRU) {
             const uint32_t w = h.lru_width, bw = w / h.lru_blocks;
@@ -401,6 +415,10 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             run_linear(e, p);
         }
         } // latent attention
+        if (forked) { // the first mixer is on its way: the main stream goes on with the second and meets it in front of the out projections
+            if (hipEventRecord(S.side_join, S.side) != hipSuccess && e.st == UZU_OK) set_error("engine: recording the side stream's join failed"), e.st = UZU_ERR_HIP;
+            s = main_stream, e.s = main_stream;
+        }
         if (h.pair_mixer) { // the second mixer beside the first: a delta rule with a decay per head and key channel, reading the same rows
             const uint32_t Hd = h.dn_num_heads, Gd = h.dn_num_groups, dk = h.dn_head_dim, dv = h.dn_value_head_dim, taps = h.dn_kernel_size, ldi = L.in_proj.n;
             const uint32_t conv_dim = 2 * Gd * dk + Hd * dv, b_col = conv_dim, a_col = b_col + Hd, g_col = a_col + h.dn_decay_rank;
@@ -427,6 +445,7 @@ uzu_status s32_encode(uzu_hip_model* m, const std::vector<uint32_t>& counts, con
             k::HeadNormGateParams np{};
             np.x = S.dn_o, np.ldx = Hd * dv, np.weight = L.dn_norm, np.gate = S.dn_gate, np.ldgate = Hd * dv, np.gate_sigmoid = 1, np.eps = h.dn_norm_epsilon, np.rows = rows, np.heads = Hd, np.width = dv;
             RUN("head_norm_gate_rows", (size_t)rows * Hd * dv * 12, k::head_norm_gate_rows(s, np));
+            if (forked && hipStreamWaitEvent(main_stream, S.side_join, 0) != hipSuccess && e.st == UZU_OK) set_error("engine: waiting for the side stream failed"), e.st = UZU_ERR_HIP;
             // tmp = scale_main * out(main) + scale_second * out(second)
             // (a scale of exactly zero takes its mixer's product out; both zero: a product that vanishes)
             const bool main_on = h.pair_scale_main != 0.0f, second_on = h.pair_scale_second != 0.0f;
@@ -993,6 +1012,11 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(void*), &p)); S.d_cache2_ptrs = (void**)p;
     TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_shift_ptrs = (float**)p;
     if (any_pair) {
+        if (hipStreamCreateWithFlags(&S.side, hipStreamNonBlocking) != hipSuccess || hipEventCreateWithFlags(&S.side_fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&S.side_join, hipEventDisableTiming) != hipSuccess) {
+            set_error("model_create: the side stream of a pair of mixers could not be created");
+            return fail(UZU_ERR_HIP);
+        }
         TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_pair_state_ptrs = (float**)p;
         TRY(dev_alloc(m, (size_t)nl * S.max_seqs * sizeof(float*), &p)); S.d_pair_conv_ptrs = (float**)p;
     }
@@ -1038,6 +1062,12 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
 }
 
 void s32_destroy(uzu_hip_model* m) {
+    if (m->s32->side) {
+        (void)hipStreamSynchronize(m->s32->side);
+        (void)hipStreamDestroy(m->s32->side);
+    }
+    if (m->s32->side_fork) (void)hipEventDestroy(m->s32->side_fork);
+    if (m->s32->side_join) (void)hipEventDestroy(m->s32->side_join);
     delete m->s32;
     m->s32 = nullptr;
 }

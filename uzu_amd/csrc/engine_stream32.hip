@@ -22,6 +22,12 @@
 // key part for all heads (interleaved pairs, scaled frequencies) with a sigmoid gate per head, per-head query / key norms on the cached-key attention, and a
 // gated linear recurrent unit behind a short convolution (k_gated_lru.hip).
 //
+// A fourth family (Zovolorn) adds: sublayers WITHOUT a norm in front that read the stream through a short causal convolution (rows + convolution, the window is
+// sequence state; k_causal_conv.hip) and join it behind an RMS norm taken in equal parts of the row, a hashed (previous token, token) table beside the embedding, a
+// capped read-out, a gelu-gated dense block with biases; on the cached-key attention one RMS norm over the whole query / key projection, interleaved pairs, a sigmoid
+// gate per head, causal chunks, values that are the key rows, a temperature per head and a learned bias per distance bucket; and a SECOND mixer beside the first in one
+// layer -- a gated delta rule with a decay per head and key channel (k_channel_delta.hip) -- whose result is summed with the first's through their own out projections.
+//
 // Precisions: `bf16_products` (default) rounds the activation operand of every matrix product to bf16 and keeps the latent cache in bf16; UZU_MODEL_FULL_F32
 // makes every product a true f32 product and the cache f32.  Everything else is f32 either way.
 #include <algorithm>

@@ -107,6 +107,7 @@ MECHANISMS = {
     "delta_rule_wide": one_layer(pair(d_heads=1, d_kv_heads=1, d_dim=33, d_vdim=70, conv=4, rank=9, left_scale=0.0)),
     "delta_rule_keys_of_130": one_layer(pair(d_heads=2, d_kv_heads=2, d_dim=130, d_vdim=4, conv=1, left_scale=0.0)),
     "delta_rule_keys_of_100": one_layer(pair(d_heads=2, d_kv_heads=1, d_dim=100, d_vdim=20, conv=3, left_scale=0.0)),
+    "delta_rule_unequal_low_ranks": one_layer(pair(rank=2, gate_rank=5, left_scale=0.0)),
     "pair_with_dense_block": one_layer(pair(mlp=O.dense(24), left_scale=0.6, right_scale=0.9)),
     "one_tap": one_layer(O.attention_layer(2, 1, 8, 8, rot_dims=4, mlp=O.dense(16)), taps=1),
     "five_taps": one_layer(O.attention_layer(2, 1, 8, 8, rot_dims=4, mlp=O.dense(16)), taps=5),
@@ -489,7 +490,7 @@ def random_config(seed):
             G, Gd = pick(1, 2, 3), pick(1, 2)
             rows = pick(1, 2, 5, 8, 32)
             layers.append(O.parallel_layer(G * pick(1, 2), G, pick(8, 16, 24, 64), pick(1, 6, 32, 64, 100), rows, pick(rows / 2 + 0.5, rows + 3.0, 240.0), Gd * pick(1, 2, 3), Gd,
-                                           pick(4, 16, 32, 40), pick(8, 16, 64, 80), pick(1, 2, 3, 4), rank=pick(1, 4, 24), scale=pick(0.1, 0.2, 0.35),
+                                           pick(4, 16, 32, 40), pick(8, 16, 64, 80), pick(1, 2, 3, 4), rank=pick(1, 4, 24), gate_rank=pick(None, 2, 7), scale=pick(0.1, 0.2, 0.35),
                                            left_scale=pick(0.3, 0.6, 1.0), right_scale=pick(0.4, 0.9, 1.0), mlp=mlp))
     groups = pick(*[g for g in (1, 2, 4, 8) if width % g == 0])
     return O.config(vocab=pick(50, 257, 640), width=width, layers=layers, eps=pick(1e-6, 1e-5, 1e-3), groups=groups, taps=pick(1, 2, 3, 4), embed_scale=pick(0.5, 1.0, 4.0),

@@ -76,7 +76,7 @@ def test_oracle_delta_rule_and_sink():
 
 def cfg_full():
     return O.config(vocab=37, width=24, eps=1e-4, groups=3, taps=3, embed_scale=0.5, bigram=(19, 5, 3), logit_softcap=8.0, layers=[
-        O.parallel_layer(4, 2, 6, 10, 7, 25.0, 4, 2, 5, 3, 2, rank=3, scale=0.3, left_scale=0.6, right_scale=0.9, mlp=O.dense(20)),
+        O.parallel_layer(4, 2, 6, 10, 7, 25.0, 4, 2, 5, 3, 2, rank=3, gate_rank=4, scale=0.3, left_scale=0.6, right_scale=0.9, mlp=O.dense(20)),
         O.attention_layer(6, 3, 4, 8, rot_dims=2, rot_base=500.0, scale=0.7, mlp=None),
         O.attention_layer(2, 2, 8, 4, rot_dims=0, mlp=O.dense(12)),
     ])
@@ -118,8 +118,8 @@ def test_reader_maps_every_branch_of_the_schema(tmp_path):
     assert p.qkv_projection.n == 4 * 6 + 2 * 6 and p.rel_bias.shape == (7, 4) and p.rel_bias_max == 25.0 and p.head_temperature.shape == (4,) and not p.qk_norm_whole
     assert p.query_norm.scales.shape == (6,) and p.sinks is None and not p.has_gate
     assert (p.dn_num_heads, p.dn_num_groups, p.dn_head_dim, p.dn_value_head_dim, p.dn_kernel_size) == (4, 2, 5, 3, 2)
-    assert p.dn_in_proj.n == 2 * 2 * 5 + 4 * 3 + 4 + 3 + 3 and p.dn_conv_weights.shape == (2 * 2 * 5 + 4 * 3, 2) and p.dn_dt_bias.shape == (20,)
-    assert (p.dn_decay_up.n, p.dn_decay_up.k, p.dn_gate_up.n, p.dn_gate_up.k) == (20, 3, 12, 3) and p.dn_norm_epsilon == pytest.approx(1e-4)
+    assert p.dn_in_proj.n == 2 * 2 * 5 + 4 * 3 + 4 + 3 + 4 and p.dn_conv_weights.shape == (2 * 2 * 5 + 4 * 3, 2) and p.dn_dt_bias.shape == (20,)
+    assert (p.dn_decay_up.n, p.dn_decay_up.k, p.dn_gate_up.n, p.dn_gate_up.k) == (20, 3, 12, 4) and p.dn_norm_epsilon == pytest.approx(1e-4)
     assert np.array_equal(p.dn_in_proj.weights[20:32], O.bf16_bits(W["l0.mix.right.v"]))  # rows q | k | v | beta | decay down | gate down
     assert np.array_equal(p.dn_in_proj.weights[36:39], O.bf16_bits(W["l0.mix.right.a1"]))
     assert p.hidden_dim == 20 and p.activation == D.ACT_GELU_APPROX and p.up_projection.n == 40 and p.up_projection.out_biases.shape == (40,) and p.post_mlp_norm.groups == 3
@@ -134,7 +134,7 @@ def test_reader_maps_every_branch_of_the_schema(tmp_path):
     assert loader.load_model_dir(write(tmp_path, cfg, spare, "spare"), max_context_length=64).layers[1].no_mlp
     d = b.desc()  # the ctypes description carries them
     assert d.bigram_buckets == 19 and d.layers[0].pair_mixer == 1 + D.MIXER_DELTA_NET and d.layers[0].rel_bias_rows == 7 and d.layers[1].qk_norm_whole == 1
-    assert d.layers[0].dn_decay_rank == 3 and d.output_norm.groups == 3 and d.logit_soft_cap == 8.0
+    assert d.layers[0].dn_decay_rank == 3 and d.layers[0].dn_gate_rank == 4 and d.output_norm.groups == 3 and d.logit_soft_cap == 8.0
     # no convolution, no table, one group, no cap
     bare = O.config(vocab=37, width=24, layers=[O.attention_layer(2, 1, 4, 4)], taps=1)
     del bare["canon"], bare["norm"]["groups"]

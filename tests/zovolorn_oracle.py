@@ -236,13 +236,14 @@ def attention_layer(heads, kv_heads, dim, vdim, rot_dims=0, rot_base=10000.0, sc
     return {"type": "attention", "mixer": mx, "mlp": mlp}
 
 
-def parallel_layer(heads, kv_heads, dim, chunk, rel_rows, bias_max, d_heads, d_kv_heads, d_dim, d_vdim, conv, rank=3, scale=None, left_scale=1.0, right_scale=1.0, mlp=None):
-    """`rel_rows` and `rank` size tensors only (a reader takes them from the shapes): they are kept under '_sizes', which a reader ignores"""
+def parallel_layer(heads, kv_heads, dim, chunk, rel_rows, bias_max, d_heads, d_kv_heads, d_dim, d_vdim, conv, rank=3, scale=None, left_scale=1.0, right_scale=1.0, mlp=None, gate_rank=None):
+    """`rel_rows`, `rank` (of the decay's two factors) and `gate_rank` (of the gate's; default: the same) size tensors only (a reader takes them from the shapes):
+    they are kept under '_sizes', which a reader ignores"""
     left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "mask": {"size": int(chunk)}, "bias_max": float(bias_max),
             "scale": float(scale if scale is not None else dim ** -0.5)}
     right = {"heads": d_heads, "kv_heads": d_kv_heads, "dim": d_dim, "vdim": d_vdim, "conv": int(conv)}
     return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": float(left_scale), "right_scale": float(right_scale)}, "mlp": mlp,
-            "_sizes": {"rel_rows": int(rel_rows), "rank": int(rank)}}
+            "_sizes": {"rel_rows": int(rel_rows), "rank": int(rank), "gate_rank": int(gate_rank if gate_rank is not None else rank)}}
 
 
 def config(vocab, width, layers, eps=1e-5, groups=1, taps=4, embed_scale=1.0, bigram=None, logit_softcap=0.0):
@@ -304,7 +305,7 @@ def weights(cfg, seed):
             lin(q + "q", Gd * dk, width, 2.0), lin(q + "k", Gd * dk, width, 2.0), lin(q + "v", Hd * dv, width, 1.5), lin(q + "b", Hd, width, 2.0)
             for n, ch in (("q", Gd * dk), ("k", Gd * dk), ("v", Hd * dv)):
                 W[q + n + ".conv"] = to_bf16(rng.standard_normal((ch, ct)) * 0.6)
-            lin(q + "a1", rank, width), lin(q + "a2", Hd * dk, rank, 2.0), lin(q + "g1", rank, width), lin(q + "g2", Hd * dv, rank, 2.0)
+            lin(q + "a1", rank, width), lin(q + "a2", Hd * dk, rank, 2.0), lin(q + "g1", sz["gate_rank"], width), lin(q + "g2", Hd * dv, sz["gate_rank"], 2.0)
             vec(q + "A_log", Hd, -1.0, 3.0), vec(q + "dt_bias", Hd * dk, -1.0, 3.0), vec(q + "norm", dv, 1.0, 0.6)
             lin(q + "o", width, Hd * dv)
         if lc.get("mlp") is not None:

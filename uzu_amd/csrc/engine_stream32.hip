@@ -850,7 +850,8 @@ uzu_status s32_create(uzu_hip_context* ctx, const uzu_model_desc* desc, uint32_t
             if (h.head_temperature) TRY(upload(m, h.head_temperature, (size_t)h.num_heads * 4, &X.head_temp));
             if (h.rel_bias_rows) { // the bias by distance: the bucket rule once, in double, for every distance up to the one the last bucket starts at
                 const uint32_t B = h.rel_bias_rows, E = B / 2, H = h.num_heads;
-                const uint32_t far = B == 1 ? 0u : (uint32_t)ceil((double)h.rel_bias_max);
+                // (distances beyond the last bucket's start share its row; no distance reaches the cache's capacity)
+                const uint32_t far = B == 1 ? 0u : (uint32_t)std::min<double>(ceil((double)h.rel_bias_max), (double)m->max_positions);
                 std::vector<float> tab((size_t)(far + 1) * H);
                 for (uint32_t n = 0; n <= far; ++n) {
                     uint32_t b = n;
